@@ -1,0 +1,445 @@
+// Decode-step self-attention kernels for gfx950 (MI355X): wave64, 128-bit coalesced K/V loads,
+// DPP row reductions, online softmax per lane-group, split along the context axis.
+//
+// Replaces the kernel sequence of FasterLLaMA's generation branch
+// (fasterLlama/cuda/open_decoder.cu:138-239): RoPE (decoder_kernels.cu:425-464), V pass-through
+// (:858-884), cache append (:597-632), Q K^T GEMV, block softmax (:800-835) and P V GEMV.
+//
+// Work decomposition
+//   grid = (nsplit, H, B); one workgroup streams `chunk` consecutive cache rows of one (b, h).
+//   A row of D elements is 16-byte chunks; LPR = min(64, D*sizeof(T)/16) lanes own one row, so a
+//   wave covers 64/LPR rows per load instruction and every load instruction of a workgroup
+//   touches one contiguous span of the cache.  Each lane-group keeps a private online-softmax
+//   state (m, l, o[its dims]); the groups of a workgroup are merged through LDS at the end.
+//   With nsplit == 1 the merged result is normalised and written to `out`; otherwise the
+//   unnormalised (m, l, o[D]) partial goes to the workspace for the combine kernel.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace flattn {
+
+struct Params {
+    const void *q, *k_new, *v_new;
+    void *k_cache, *v_cache;
+    const float *freq_cis;
+    const float *attn_mask;
+    const int32_t *pos_per_seq;
+    float *out;
+    float *part_o; // [B*H, split_cap, D]
+    float *part_m; // [B*H, split_cap]
+    float *part_l; // [B*H, split_cap]
+    const float *inp_scale, *wq_scale, *wk_scale, *wv_scale;
+    int8_t *out_int8;
+    float *out_scale;
+    int64_t mask_ld;
+    int32_t B, H, L;
+    int32_t start_pos, rope_row;
+    int32_t chunk;     // cache rows per split
+    int32_t split_cap; // stride of the partial arrays along the split axis
+    int32_t direct;    // 1: single split, write normalised output straight to `out`
+    float scale;
+};
+
+constexpr float kMaxFloor = -1e9f; // reference: float max_val = -1e9f (decoder_kernels.cu:811)
+
+// ---------------------------------------------------------------- lane-group reductions (DPP)
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x)
+{
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over the LPR consecutive lanes that share a cache row; every lane gets the same bits.
+template <int LPR>
+__device__ __forceinline__ float group_sum(float x)
+{
+    if constexpr (LPR >= 2) x += dpp_move<0xB1>(x);  // quad_perm [1,0,3,2]
+    if constexpr (LPR >= 4) x += dpp_move<0x4E>(x);  // quad_perm [2,3,0,1]
+    if constexpr (LPR >= 8) x += dpp_move<0x141>(x); // row_half_mirror
+    if constexpr (LPR >= 16) x += dpp_move<0x140>(x); // row_mirror
+    if constexpr (LPR >= 32) x += __shfl_xor(x, 16);
+    if constexpr (LPR >= 64) x += __shfl_xor(x, 32);
+    return x;
+}
+
+__device__ __forceinline__ float wave_max(float x)
+{
+    x = fmaxf(x, dpp_move<0xB1>(x));
+    x = fmaxf(x, dpp_move<0x4E>(x));
+    x = fmaxf(x, dpp_move<0x141>(x));
+    x = fmaxf(x, dpp_move<0x140>(x));
+    x = fmaxf(x, __shfl_xor(x, 16));
+    x = fmaxf(x, __shfl_xor(x, 32));
+    return x;
+}
+
+// ---------------------------------------------------------------- 16-byte element vectors
+
+template <typename T> struct Vec16;
+template <> struct Vec16<float> {
+    static constexpr int N = 4;
+    typedef float type __attribute__((ext_vector_type(4)));
+};
+template <> struct Vec16<_Float16> {
+    static constexpr int N = 8;
+    typedef _Float16 type __attribute__((ext_vector_type(8)));
+};
+
+// RoPE of one interleaved pair; the operation order is part of the contract with the CPU
+// checker so that the appended cache row is bit-identical:
+//   o0 = fma(x0, c, -(x1*s)),  o1 = fma(x1, c, x0*s)      (decoder_kernels.cu:455-458)
+__device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, float &o0, float &o1)
+{
+    float t0 = __fmul_rn(x1, s);
+    float t1 = __fmul_rn(x0, s);
+    o0 = __fmaf_rn(x0, c, -t0);
+    o1 = __fmaf_rn(x1, c, t1);
+}
+
+// float -> storage type in two separately rounded steps (fp32 result first, then nearest-even to
+// the storage type).  The empty asm keeps the compiler from folding the conversion into a
+// mixed-precision FMA that would round the exact product-sum straight to half.
+template <typename T>
+__device__ __forceinline__ T to_storage(float x)
+{
+    asm volatile("" : "+v"(x));
+    return (T)x;
+}
+
+// Loads VEC consecutive elements of a [B,1,H,D] operand as float: storage dtype, or int32
+// accumulators scaled by inp_scale[b] * w_scale[h*D + d] (decoder_kernels.cu:449-452).
+template <typename T, int VEC>
+__device__ __forceinline__ void load_token_chunk(const void *base, size_t elem_off, bool is_i32,
+                                                 float inp_scale, const float *w_scale_at,
+                                                 float (&dst)[VEC])
+{
+    if (is_i32) {
+        const int32_t *p = reinterpret_cast<const int32_t *>(base) + elem_off;
+#pragma unroll
+        for (int i = 0; i < VEC; i += 4) {
+            int4 a = *reinterpret_cast<const int4 *>(p + i);
+            float4 w = *reinterpret_cast<const float4 *>(w_scale_at + i);
+            dst[i + 0] = __fmul_rn(__fmul_rn((float)a.x, inp_scale), w.x);
+            dst[i + 1] = __fmul_rn(__fmul_rn((float)a.y, inp_scale), w.y);
+            dst[i + 2] = __fmul_rn(__fmul_rn((float)a.z, inp_scale), w.z);
+            dst[i + 3] = __fmul_rn(__fmul_rn((float)a.w, inp_scale), w.w);
+        }
+    } else {
+        typedef typename Vec16<T>::type V;
+        V v = *reinterpret_cast<const V *>(reinterpret_cast<const T *>(base) + elem_off);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) dst[i] = (float)v[i];
+    }
+}
+
+// ---------------------------------------------------------------- streaming (split) kernel
+
+template <typename T, int D, int WAVES, int UNROLL>
+__global__ __launch_bounds__(WAVES * 64) void decode_attn_split_kernel(const Params p)
+{
+    typedef typename Vec16<T>::type V;
+    constexpr int VEC = Vec16<T>::N;
+    constexpr int CH = D / VEC;             // 16-byte chunks per row
+    constexpr int LPR = CH < 64 ? CH : 64;  // lanes per row
+    constexpr int CPL = CH / LPR;           // chunks per lane
+    constexpr int GPW = 64 / LPR;           // rows per wave per load instruction
+    constexpr int GROUPS = WAVES * GPW;     // rows per workgroup per load instruction
+    constexpr int EPL = CPL * VEC;          // elements of a row owned by one lane
+    static_assert(CH * VEC == D && LPR * CPL == CH, "head size must tile into 16-byte chunks");
+
+    __shared__ float s_o[GROUPS][D];
+    __shared__ float s_m[GROUPS];
+    __shared__ float s_l[GROUPS];
+
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int H = p.H, L = p.L;
+    const int bh = b * H + h;
+    const int P = p.pos_per_seq ? p.pos_per_seq[b] : p.start_pos;
+    const int tid = threadIdx.x;
+
+    if (P < 0 || P >= L) { // position outside the cache: store nothing, poison the output
+        if (p.direct && split == 0)
+            for (int d = tid; d < D; d += WAVES * 64) p.out[(size_t)bh * D + d] = __builtin_nanf("");
+        return;
+    }
+    const int ctx = P + 1;
+    const int start = split * p.chunk;
+    if (start >= ctx) return;
+    const int end = min(start + p.chunk, ctx);
+    const bool owns_new = (end == ctx);           // exactly one split per (b,h)
+    const int cache_end = owns_new ? P : end;     // rows [start, cache_end) come from the cache
+
+    const int lane = tid & 63, wave = tid >> 6;
+    const int g = lane / LPR, lig = lane % LPR;
+    const int group = wave * GPW + g;
+
+    const bool is_i32 = p.inp_scale != nullptr;
+    const float inp_scale = is_i32 ? p.inp_scale[b] : 0.f;
+    const int rope_row = p.rope_row < 0 ? P : p.rope_row;
+    const float *freq = p.freq_cis + (size_t)rope_row * D;
+
+    // RoPE(q) for the dims this lane owns, kept in registers (fp32)
+    float qr[EPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+        const int e0 = (c * LPR + lig) * VEC;
+        float x[VEC];
+        load_token_chunk<T, VEC>(p.q, (size_t)bh * D + e0, is_i32, inp_scale,
+                                 is_i32 ? p.wq_scale + h * D + e0 : nullptr, x);
+#pragma unroll
+        for (int i = 0; i < VEC; i += 4) {
+            float4 f = *reinterpret_cast<const float4 *>(freq + e0 + i);
+            rope_pair(x[i], x[i + 1], f.x, f.y, qr[c * VEC + i], qr[c * VEC + i + 1]);
+            rope_pair(x[i + 2], x[i + 3], f.z, f.w, qr[c * VEC + i + 2], qr[c * VEC + i + 3]);
+        }
+    }
+
+    const T *Kb = reinterpret_cast<const T *>(p.k_cache) + (size_t)bh * L * D;
+    const T *Vb = reinterpret_cast<const T *>(p.v_cache) + (size_t)bh * L * D;
+    const float *mrow = p.attn_mask ? p.attn_mask + (size_t)P * p.mask_ld : nullptr;
+    const float scale = p.scale;
+
+    float m = kMaxFloor, l = 0.f;
+    float o[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) o[e] = 0.f;
+
+    // One tile = UNROLL rows per lane-group.  CHECK guards the ragged last tile.
+    auto tile = [&](int r0, auto check_tag) {
+        constexpr bool CHECK = decltype(check_tag)::value;
+        V kv[UNROLL][CPL], vv[UNROLL][CPL];
+        float mk[UNROLL];
+        bool ok[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int row = r0 + u * GROUPS + group;
+            ok[u] = !CHECK || row < cache_end;
+            if (CHECK && !ok[u]) row = r0; // any valid row; its data is discarded
+            const T *kp = Kb + (size_t)row * D + lig * VEC;
+#pragma unroll
+            for (int c = 0; c < CPL; ++c)
+                kv[u][c] = __builtin_nontemporal_load(reinterpret_cast<const V *>(kp + c * LPR * VEC));
+            mk[u] = mrow ? mrow[row] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            int row = r0 + u * GROUPS + group;
+            if (CHECK && !ok[u]) row = r0;
+            const T *vp = Vb + (size_t)row * D + lig * VEC;
+#pragma unroll
+            for (int c = 0; c < CPL; ++c)
+                vv[u][c] = __builtin_nontemporal_load(reinterpret_cast<const V *>(vp + c * LPR * VEC));
+        }
+        float s[UNROLL];
+        float tmax = m;
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            float acc = 0.f;
+#pragma unroll
+            for (int c = 0; c < CPL; ++c)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc = fmaf((float)kv[u][c][i], qr[c * VEC + i], acc);
+            acc = group_sum<LPR>(acc);
+            s[u] = fmaf(acc, scale, mk[u]); // v = qk*scaler + mask (decoder_kernels.cu:815)
+            if (CHECK && !ok[u]) s[u] = -__builtin_inff();
+            tmax = fmaxf(tmax, s[u]);
+        }
+        const float alpha = expf(m - tmax);
+        m = tmax;
+        l *= alpha;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) o[e] *= alpha;
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (CHECK && !ok[u]) continue;
+            const float pr = expf(s[u] - m);
+            l += pr;
+#pragma unroll
+            for (int c = 0; c < CPL; ++c)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i)
+                    o[c * VEC + i] = fmaf(pr, (float)vv[u][c][i], o[c * VEC + i]);
+        }
+    };
+
+    constexpr int ROWS_PER_TILE = GROUPS * UNROLL;
+    int r = start;
+    for (; r + ROWS_PER_TILE <= cache_end; r += ROWS_PER_TILE) tile(r, std::false_type{});
+    if (r < cache_end) tile(r, std::true_type{});
+
+    // The new token: RoPE(k_new) and v_new are rounded to the storage type, appended at row P
+    // (decoder_kernels.cu:605-610) and attended to from registers.  Every group of wave 0
+    // evaluates the row (keeps the wave convergent for the DPP reduction); group 0 applies it.
+    if (owns_new && wave == 0) {
+        T *kdst = reinterpret_cast<T *>(p.k_cache) + ((size_t)bh * L + P) * D;
+        T *vdst = reinterpret_cast<T *>(p.v_cache) + ((size_t)bh * L + P) * D;
+        float kf[EPL], vf[EPL];
+        float acc = 0.f;
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+            const int e0 = (c * LPR + lig) * VEC;
+            float kx[VEC], vx[VEC];
+            load_token_chunk<T, VEC>(p.k_new, (size_t)bh * D + e0, is_i32, inp_scale,
+                                     is_i32 ? p.wk_scale + h * D + e0 : nullptr, kx);
+            load_token_chunk<T, VEC>(p.v_new, (size_t)bh * D + e0, is_i32, inp_scale,
+                                     is_i32 ? p.wv_scale + h * D + e0 : nullptr, vx);
+            V kt, vt;
+#pragma unroll
+            for (int i = 0; i < VEC; i += 4) {
+                float4 f = *reinterpret_cast<const float4 *>(freq + e0 + i);
+                float r0, r1, r2, r3;
+                rope_pair(kx[i], kx[i + 1], f.x, f.y, r0, r1);
+                rope_pair(kx[i + 2], kx[i + 3], f.z, f.w, r2, r3);
+                kt[i] = to_storage<T>(r0); kt[i + 1] = to_storage<T>(r1);
+                kt[i + 2] = to_storage<T>(r2); kt[i + 3] = to_storage<T>(r3);
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                vt[i] = to_storage<T>(vx[i]);
+                kf[c * VEC + i] = (float)kt[i];
+                vf[c * VEC + i] = (float)vt[i];
+                acc = fmaf(kf[c * VEC + i], qr[c * VEC + i], acc);
+            }
+            if (g == 0) {
+                *reinterpret_cast<V *>(kdst + e0) = kt;
+                *reinterpret_cast<V *>(vdst + e0) = vt;
+            }
+        }
+        acc = group_sum<LPR>(acc);
+        if (g == 0) {
+            const float s = fmaf(acc, scale, mrow ? mrow[P] : 0.f);
+            const float m_new = fmaxf(m, s);
+            const float alpha = expf(m - m_new);
+            const float pr = expf(s - m_new);
+            m = m_new;
+            l = fmaf(l, alpha, pr);
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) o[e] = fmaf(o[e], alpha, pr * vf[e]);
+        }
+    }
+
+    // Merge the lane-groups of the workgroup.
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+        const int e0 = (c * LPR + lig) * VEC;
+#pragma unroll
+        for (int i = 0; i < VEC; i += 4)
+            *reinterpret_cast<float4 *>(&s_o[group][e0 + i]) =
+                make_float4(o[c * VEC + i], o[c * VEC + i + 1], o[c * VEC + i + 2], o[c * VEC + i + 3]);
+    }
+    if (lig == 0) {
+        s_m[group] = m;
+        s_l[group] = l;
+    }
+    __syncthreads();
+
+    for (int d = tid; d < D; d += WAVES * 64) {
+        float M = kMaxFloor;
+#pragma unroll
+        for (int k = 0; k < GROUPS; ++k) M = fmaxf(M, s_m[k]);
+        float Lsum = 0.f, O = 0.f;
+#pragma unroll
+        for (int k = 0; k < GROUPS; ++k) {
+            const float w = expf(s_m[k] - M);
+            Lsum = fmaf(s_l[k], w, Lsum);
+            O = fmaf(s_o[k][d], w, O);
+        }
+        if (p.direct) {
+            p.out[(size_t)bh * D + d] = O / Lsum; // p = e / sum (decoder_kernels.cu:833)
+        } else {
+            const size_t slot = (size_t)bh * p.split_cap + split;
+            p.part_o[slot * D + d] = O;
+            if (d == 0) {
+                p.part_m[slot] = M;
+                p.part_l[slot] = Lsum;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- combine kernels
+
+// Merged, normalised attention output element d of (b,h) from its split partials.
+__device__ __forceinline__ float merge_partials(const Params &p, int bh, int nsp, int D, int d)
+{
+    const size_t slot0 = (size_t)bh * p.split_cap;
+    float M = kMaxFloor;
+    for (int s = 0; s < nsp; ++s) M = fmaxf(M, p.part_m[slot0 + s]);
+    float Lsum = 0.f, O = 0.f;
+    for (int s = 0; s < nsp; ++s) {
+        const float w = expf(p.part_m[slot0 + s] - M);
+        Lsum = fmaf(p.part_l[slot0 + s], w, Lsum);
+        O = fmaf(p.part_o[(slot0 + s) * D + d], w, O);
+    }
+    return O / Lsum;
+}
+
+// grid = B*H, block = min(D, 256): out[b, h*D + d] from the partials of (b,h).
+__global__ void decode_attn_combine_kernel(const Params p, int D)
+{
+    const int bh = blockIdx.x;
+    const int b = bh / p.H;
+    const int P = p.pos_per_seq ? p.pos_per_seq[b] : p.start_pos;
+    const bool bad = (P < 0 || P >= p.L);
+    const int nsp = bad ? 0 : (P + p.chunk) / p.chunk; // ceil((P+1)/chunk)
+    for (int d = threadIdx.x; d < D; d += blockDim.x)
+        p.out[(size_t)bh * D + d] = bad ? __builtin_nanf("") : merge_partials(p, bh, nsp, D, d);
+}
+
+// grid = B, block = 1024: merge + per-row absmax INT8 quantisation over the H*D outputs of one
+// sequence (launchAttnQuantizedTransposeKernel, decoder_kernels.cu:1179-1212, seq_len == 1):
+//   absmax = max(-1e9, max |x|); scale[b] = absmax/127; q = sat_s8(rint(x*127/absmax)).
+__global__ __launch_bounds__(1024) void decode_attn_combine_quant_kernel(const Params p, int D)
+{
+    __shared__ float s_red[16];
+    const int b = blockIdx.x;
+    const int HD = p.H * D;
+    const int P = p.pos_per_seq ? p.pos_per_seq[b] : p.start_pos;
+    const bool bad = (P < 0 || P >= p.L);
+    const int nsp = bad ? 0 : (P + p.chunk) / p.chunk;
+    const float nan = __builtin_nanf("");
+
+    float absmax = kMaxFloor;
+    for (int e = threadIdx.x; e < HD; e += blockDim.x) {
+        const float x = bad ? nan : merge_partials(p, b * p.H + e / D, nsp, D, e % D);
+        if (p.out) p.out[(size_t)b * HD + e] = x;
+        absmax = fmaxf(absmax, fabsf(x));
+    }
+    absmax = wave_max(absmax);
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = absmax;
+    __syncthreads();
+    absmax = s_red[0];
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) absmax = fmaxf(absmax, s_red[w]);
+    if (threadIdx.x == 0) p.out_scale[b] = absmax / 127.0f;
+
+    for (int e = threadIdx.x; e < HD; e += blockDim.x) {
+        const float x = bad ? nan : merge_partials(p, b * p.H + e / D, nsp, D, e % D);
+        const float v = rintf(__fmul_rn(x, 127.0f) / absmax);
+        const int qv = (v != v) ? 0 : (int)fminf(fmaxf(v, -128.f), 127.f);
+        p.out_int8[(size_t)b * HD + e] = (int8_t)qv;
+    }
+}
+
+// ---------------------------------------------------------------- RoPE table producer
+
+// freq_cis[r, 2i] = cos(r * base^(-2i/D)), freq_cis[r, 2i+1] = sin(same); evaluated in double
+// and rounded once (the reference uses __powf/__cosf/__sinf, decoding_kernels.cu:100-114).
+__global__ void rope_table_kernel(float *table, int rows, int D, double base)
+{
+    const int half = D >> 1;
+    const int64_t n = (int64_t)rows * half;
+    for (int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; t < n;
+         t += (int64_t)gridDim.x * blockDim.x) {
+        const int r = (int)(t / half), i = (int)(t % half);
+        const double theta = (double)r * pow(base, -2.0 * (double)i / (double)D);
+        double sn, cs;
+        sincos(theta, &sn, &cs);
+        *reinterpret_cast<float2 *>(table + (size_t)r * D + 2 * i) = make_float2((float)cs, (float)sn);
+    }
+}
+
+} // namespace flattn

@@ -1,0 +1,326 @@
+// C ABI of the decode-step attention library (see include/fl_decode_attn.h).
+// Host side: argument validation, launch planning and kernel dispatch.  Enqueue-only: no
+// allocation, no synchronisation, no state kept between calls.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <type_traits>
+
+#include "../../include/fl_decode_attn.h"
+#include "decode_attn_kernels.hpp"
+
+namespace {
+
+using flattn::Params;
+
+thread_local int g_last_hip_error = 0;
+
+constexpr int kWaves = 4;        // 256 threads per streaming workgroup
+constexpr int kMinChunkRows = 64; // never split a context finer than this
+constexpr int kMaxSplits = 1024;
+
+inline bool check_hip(hipError_t e)
+{
+    if (e != hipSuccess) {
+        g_last_hip_error = (int)e;
+        return false;
+    }
+    return true;
+}
+
+// Compute units of the current device, cached per device id.
+int device_cus()
+{
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+bool head_dim_ok(int D)
+{
+    return D == 32 || D == 64 || D == 128 || D == 256 || D == 512 || D == 1024;
+}
+
+int validate_desc(const fl_attn_desc *d)
+{
+    if (!d) return FL_ATTN_ERR_NULL_POINTER;
+    if (d->dtype != FL_ATTN_F32 && d->dtype != FL_ATTN_F16) return FL_ATTN_ERR_DTYPE;
+    if (d->batch_size <= 0 || d->head_num <= 0 || d->total_len <= 0) return FL_ATTN_ERR_SHAPE;
+    if (d->batch_size > 65535 || d->head_num > 65535) return FL_ATTN_ERR_SHAPE; // grid y/z limits
+    if (!head_dim_ok(d->size_per_head)) return FL_ATTN_ERR_HEAD_DIM;
+    if (d->nsplit < 0 || d->nsplit > kMaxSplits || d->reserved != 0) return FL_ATTN_ERR_ARGUMENT;
+    if (!(d->softmax_scale >= 0.f) || std::isinf(d->softmax_scale)) return FL_ATTN_ERR_ARGUMENT;
+    // element counts of a cache must stay addressable with a 64-bit byte offset; B*H must fit int
+    if ((int64_t)d->batch_size * d->head_num > (int64_t)INT32_MAX / 2) return FL_ATTN_ERR_SHAPE;
+    return FL_ATTN_OK;
+}
+
+// Rows a streaming workgroup consumes per loop trip; chunk sizes are multiples of it.
+int rows_per_tile(const fl_attn_desc *d, int unroll)
+{
+    const int vec = d->dtype == FL_ATTN_F16 ? 8 : 4;
+    const int ch = d->size_per_head / vec;
+    const int lpr = ch < 64 ? ch : 64;
+    return kWaves * (64 / lpr) * unroll;
+}
+
+int unroll_for(const fl_attn_desc *d)
+{
+    const int vec = d->dtype == FL_ATTN_F16 ? 8 : 4;
+    const int ch = d->size_per_head / vec;
+    const int cpl = ch <= 64 ? 1 : ch / 64;
+    return cpl >= 4 ? 1 : (cpl == 2 ? 2 : 4);
+}
+
+// Upper bound of splits for any context of this shape: sizes the workspace.
+int split_cap(const fl_attn_desc *d)
+{
+    if (d->nsplit > 0) return d->nsplit;
+    const int64_t bh = (int64_t)d->batch_size * d->head_num;
+    const int64_t target = (int64_t)device_cus() * 8;
+    int64_t want = (target + bh - 1) / bh;
+    int64_t most = ((int64_t)d->total_len + kMinChunkRows - 1) / kMinChunkRows;
+    int64_t n = want < most ? want : most;
+    if (n < 1) n = 1;
+    if (n > kMaxSplits) n = kMaxSplits;
+    return (int)n;
+}
+
+void make_plan(const fl_attn_desc *d, int ctx, fl_attn_plan *plan)
+{
+    const int tile = rows_per_tile(d, unroll_for(d));
+    int n;
+    if (d->nsplit > 0) {
+        n = d->nsplit;
+    } else {
+        const int64_t bh = (int64_t)d->batch_size * d->head_num;
+        const int64_t target = (int64_t)device_cus() * 8;
+        int64_t want = (target + bh - 1) / bh;
+        int64_t most = ((int64_t)ctx + kMinChunkRows - 1) / kMinChunkRows;
+        int64_t nn = want < most ? want : most;
+        if (nn < 1) nn = 1;
+        if (nn > kMaxSplits) nn = kMaxSplits;
+        n = (int)nn;
+    }
+    if (n > ctx) n = ctx > 0 ? ctx : 1;
+    int chunk = (ctx + n - 1) / n;
+    if (d->nsplit == 0) chunk = (chunk + tile - 1) / tile * tile; // whole tiles per split
+    if (chunk < 1) chunk = 1;
+    plan->chunk_rows = chunk;
+    plan->nsplit = (ctx + chunk - 1) / chunk;
+    plan->threads = kWaves * 64;
+    plan->two_pass = plan->nsplit > 1;
+}
+
+size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+size_t workspace_need(const fl_attn_desc *d)
+{
+    const size_t slots = (size_t)d->batch_size * d->head_num * (size_t)split_cap(d);
+    const size_t part_o = align_up(slots * d->size_per_head * sizeof(float), 256);
+    const size_t part_ml = align_up(slots * sizeof(float), 256);
+    return part_o + 2 * part_ml;
+}
+
+template <typename T, int D>
+hipError_t launch_split(const Params &p, dim3 grid, hipStream_t stream)
+{
+    constexpr int VEC = flattn::Vec16<T>::N;
+    constexpr int CH = D / VEC;
+    constexpr int CPL = CH <= 64 ? 1 : CH / 64;
+    constexpr int UNROLL = CPL >= 4 ? 1 : (CPL == 2 ? 2 : 4);
+    hipLaunchKernelGGL((flattn::decode_attn_split_kernel<T, D, kWaves, UNROLL>), grid, dim3(kWaves * 64), 0,
+                       stream, p);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t dispatch_split(int D, const Params &p, dim3 grid, hipStream_t stream)
+{
+    switch (D) {
+    case 32: return launch_split<T, 32>(p, grid, stream);
+    case 64: return launch_split<T, 64>(p, grid, stream);
+    case 128: return launch_split<T, 128>(p, grid, stream);
+    case 256: return launch_split<T, 256>(p, grid, stream);
+    case 512: return launch_split<T, 512>(p, grid, stream);
+    case 1024: return launch_split<T, 1024>(p, grid, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+} // namespace
+
+extern "C" {
+
+int fl_attn_version(void) { return 100; }
+
+int fl_attn_last_hip_error(void) { return g_last_hip_error; }
+
+const char *fl_attn_strerror(int status)
+{
+    switch (status) {
+    case FL_ATTN_OK: return "ok";
+    case FL_ATTN_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case FL_ATTN_ERR_HEAD_DIM: return "invalid size_per_head (supported: 32, 64, 128, 256, 512, 1024)";
+    case FL_ATTN_ERR_SHAPE: return "invalid batch_size / head_num / total_len";
+    case FL_ATTN_ERR_POSITION: return "start_pos or rope_row out of range for total_len";
+    case FL_ATTN_ERR_WORKSPACE: return "workspace missing, too small or not 256-byte aligned";
+    case FL_ATTN_ERR_DTYPE: return "dtype must be FL_ATTN_F32 or FL_ATTN_F16";
+    case FL_ATTN_ERR_HIP: return "a HIP runtime call failed";
+    case FL_ATTN_ERR_ALIGNMENT: return "tensor base pointers must be 16-byte aligned";
+    case FL_ATTN_ERR_ARGUMENT: return "inconsistent arguments";
+    default: return "unknown status";
+    }
+}
+
+int fl_decode_attn_workspace_bytes(const fl_attn_desc *desc, size_t *bytes)
+{
+    if (!bytes) return FL_ATTN_ERR_NULL_POINTER;
+    int st = validate_desc(desc);
+    if (st != FL_ATTN_OK) return st;
+    *bytes = workspace_need(desc);
+    return FL_ATTN_OK;
+}
+
+int fl_kv_cache_bytes(const fl_attn_desc *desc, size_t *bytes)
+{
+    if (!bytes) return FL_ATTN_ERR_NULL_POINTER;
+    int st = validate_desc(desc);
+    if (st != FL_ATTN_OK) return st;
+    const size_t e = desc->dtype == FL_ATTN_F16 ? 2 : 4;
+    *bytes = (size_t)desc->batch_size * desc->head_num * (size_t)desc->total_len * desc->size_per_head * e;
+    return FL_ATTN_OK;
+}
+
+int fl_decode_attn_plan(const fl_attn_desc *desc, int32_t ctx, fl_attn_plan *plan)
+{
+    if (!plan) return FL_ATTN_ERR_NULL_POINTER;
+    int st = validate_desc(desc);
+    if (st != FL_ATTN_OK) return st;
+    if (ctx < 1 || ctx > desc->total_len) return FL_ATTN_ERR_POSITION;
+    make_plan(desc, ctx, plan);
+    return FL_ATTN_OK;
+}
+
+int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream, int passes)
+{
+    int st = validate_desc(desc);
+    if (st != FL_ATTN_OK) return st;
+    if (!io) return FL_ATTN_ERR_NULL_POINTER;
+    if ((passes & ~3) != 0 || passes == 0) return FL_ATTN_ERR_ARGUMENT;
+    if (!io->q || !io->k_new || !io->v_new || !io->k_cache || !io->v_cache || !io->freq_cis)
+        return FL_ATTN_ERR_NULL_POINTER;
+    const bool quant = io->out_int8 != nullptr;
+    if (!io->out && !quant) return FL_ATTN_ERR_NULL_POINTER;
+    if (quant && !io->out_scale) return FL_ATTN_ERR_NULL_POINTER;
+    if (io->reserved != 0) return FL_ATTN_ERR_ARGUMENT;
+    const bool i32 = io->qkv_inp_scale != nullptr;
+    if (i32 && (!io->q_weight_scale || !io->k_weight_scale || !io->v_weight_scale)) return FL_ATTN_ERR_NULL_POINTER;
+    if (!i32 && (io->q_weight_scale || io->k_weight_scale || io->v_weight_scale)) return FL_ATTN_ERR_ARGUMENT;
+    if (!aligned16(io->q) || !aligned16(io->k_new) || !aligned16(io->v_new) || !aligned16(io->k_cache) ||
+        !aligned16(io->v_cache) || !aligned16(io->freq_cis) || !aligned16(io->out) ||
+        (i32 && (!aligned16(io->q_weight_scale) || !aligned16(io->k_weight_scale) || !aligned16(io->v_weight_scale))))
+        return FL_ATTN_ERR_ALIGNMENT;
+
+    const int L = desc->total_len;
+    const bool ragged = io->start_pos_per_seq != nullptr;
+    int max_pos;
+    if (ragged) {
+        max_pos = io->max_start_pos < 0 ? L - 1 : io->max_start_pos;
+        if (max_pos >= L) return FL_ATTN_ERR_POSITION;
+    } else {
+        // reference: rows attended = start_pos + seq_len must fit the cache (open_decoder.cu:170-171)
+        if (io->start_pos < 0 || io->start_pos >= L) return FL_ATTN_ERR_POSITION;
+        max_pos = io->start_pos;
+    }
+    if (io->rope_row < FL_ATTN_ROPE_AT_POSITION) return FL_ATTN_ERR_POSITION;
+    if (io->attn_mask && io->mask_ld < 0) return FL_ATTN_ERR_ARGUMENT;
+
+    fl_attn_plan plan;
+    make_plan(desc, max_pos + 1, &plan);
+    const int cap = split_cap(desc);
+    if (plan.nsplit > cap) return FL_ATTN_ERR_ARGUMENT;
+
+    const bool direct = plan.nsplit == 1 && !quant;
+    const size_t need = workspace_need(desc);
+    if (!direct) {
+        if (!io->workspace || io->workspace_bytes < need) return FL_ATTN_ERR_WORKSPACE;
+        if ((reinterpret_cast<uintptr_t>(io->workspace) & 255u) != 0) return FL_ATTN_ERR_WORKSPACE;
+    }
+
+    const int D = desc->size_per_head;
+    Params p{};
+    p.q = io->q; p.k_new = io->k_new; p.v_new = io->v_new;
+    p.k_cache = io->k_cache; p.v_cache = io->v_cache;
+    p.freq_cis = io->freq_cis; p.attn_mask = io->attn_mask; p.pos_per_seq = io->start_pos_per_seq;
+    p.out = io->out;
+    if (!direct) {
+        const size_t slots = (size_t)desc->batch_size * desc->head_num * (size_t)cap;
+        const size_t part_o = align_up(slots * D * sizeof(float), 256);
+        const size_t part_ml = align_up(slots * sizeof(float), 256);
+        char *ws = static_cast<char *>(io->workspace);
+        p.part_o = reinterpret_cast<float *>(ws);
+        p.part_m = reinterpret_cast<float *>(ws + part_o);
+        p.part_l = reinterpret_cast<float *>(ws + part_o + part_ml);
+    }
+    p.inp_scale = io->qkv_inp_scale; p.wq_scale = io->q_weight_scale;
+    p.wk_scale = io->k_weight_scale; p.wv_scale = io->v_weight_scale;
+    p.out_int8 = io->out_int8; p.out_scale = io->out_scale;
+    p.mask_ld = io->mask_ld;
+    p.B = desc->batch_size; p.H = desc->head_num; p.L = L;
+    p.start_pos = io->start_pos; p.rope_row = io->rope_row;
+    p.chunk = plan.chunk_rows; p.split_cap = cap; p.direct = direct ? 1 : 0;
+    p.scale = desc->softmax_scale > 0.f ? desc->softmax_scale : 1.0f / sqrtf((float)D);
+
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    if (passes & 1) {
+        dim3 grid(plan.nsplit, desc->head_num, desc->batch_size);
+        hipError_t e = desc->dtype == FL_ATTN_F16 ? dispatch_split<_Float16>(D, p, grid, stream)
+                                                  : dispatch_split<float>(D, p, grid, stream);
+        if (!check_hip(e)) return FL_ATTN_ERR_HIP;
+    }
+    if ((passes & 2) && !direct) {
+        if (quant) {
+            hipLaunchKernelGGL(flattn::decode_attn_combine_quant_kernel, dim3(desc->batch_size), dim3(1024), 0,
+                               stream, p, D);
+        } else {
+            hipLaunchKernelGGL(flattn::decode_attn_combine_kernel, dim3(desc->batch_size * desc->head_num),
+                               dim3(D < 256 ? D : 256), 0, stream, p, D);
+        }
+        if (!check_hip(hipGetLastError())) return FL_ATTN_ERR_HIP;
+    }
+    return FL_ATTN_OK;
+}
+
+int fl_decode_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream)
+{
+    return fl_decode_attn_forward_passes(desc, io, hip_stream, 3);
+}
+
+int fl_rope_table(float *freq_cis, int32_t rows, int32_t size_per_head, float base, void *hip_stream)
+{
+    if (!freq_cis) return FL_ATTN_ERR_NULL_POINTER;
+    if (rows <= 0) return FL_ATTN_ERR_SHAPE;
+    if (size_per_head <= 0 || (size_per_head & 1)) return FL_ATTN_ERR_HEAD_DIM;
+    if (!(base > 0.f)) return FL_ATTN_ERR_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(freq_cis) & 7u) != 0) return FL_ATTN_ERR_ALIGNMENT;
+    const int64_t n = (int64_t)rows * (size_per_head / 2);
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 65535) blocks = 65535;
+    hipLaunchKernelGGL(flattn::rope_table_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                       static_cast<hipStream_t>(hip_stream), freq_cis, rows, size_per_head, (double)base);
+    if (!check_hip(hipGetLastError())) return FL_ATTN_ERR_HIP;
+    return FL_ATTN_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,152 @@
+/*
+ * fl_decode_attn.h — C ABI of the MI355X (gfx950) decode-step self-attention library.
+ *
+ * One call replaces the seq_len == 1 attention segment of FasterLLaMA's
+ * OpenDecoder::forward (fasterLlama/cuda/open_decoder.cu:138-239):
+ *
+ *   launchQKRoteEmbeddingTranspose      open_decoder.cu:142-146   decoder_kernels.cu:425-464
+ *   launchDequantizedVTransposeKernel   open_decoder.cu:157-158   decoder_kernels.cu:858-884
+ *   launchStoreKVcacheKernel            open_decoder.cu:170-171   decoder_kernels.cu:597-662
+ *   cublasSgemvStridedBatched (Q K^T)   open_decoder.cu:194-201
+ *   launchBlockSoftmaxKernel            open_decoder.cu:207-208   decoder_kernels.cu:800-848
+ *   cublasSgemvStridedBatched (P V)     open_decoder.cu:231-238
+ *
+ * and, optionally, the two stages on either side of it:
+ *   int32 -> float dequantisation of Q/K/V   decoder_kernels.cu:449-452, :875-878
+ *   launchAttnQuantizedTransposeKernel       open_decoder.cu:245-246  decoder_kernels.cu:1179-1300
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; the library allocates nothing and
+ *     keeps no state between calls (reference: OpenDecoder stores raw non-owning pointers,
+ *     open_decoder.cu:31-45, :360-375);
+ *   - work is only enqueued on the given hipStream_t (passed as void*); no host synchronisation;
+ *   - functions return FL_ATTN_OK or a negative fl_attn_status; they never exit() or throw
+ *     (the reference prints and exits, utils.h:50-80, or throws a const char*,
+ *     decoder_kernels.cu:588);
+ *   - sizes are 64-bit where the reference's int would overflow (open_decoder.cu:54-67).
+ *
+ * Layouts (bit-exact with the reference)
+ *   q, k_new, v_new : [B, 1, H, D]  == [B, H, 1, D] for one token  (decoder_kernels.cu:461)
+ *   k_cache, v_cache: [B, H, L, D], row of token t of (b,h) at ((b*H + h)*L + t)*D
+ *                     (decoder_kernels.cu:606-607)
+ *   freq_cis        : [rows, D] float, row r = cos/sin interleaved (decoding_kernels.cu:100-114)
+ *   attn_mask       : [L, mask_ld] float, additive; the row used is start_pos
+ *                     (open_decoder.cu:207: attn_mask + start_pos * total_len_)
+ *   out             : [B, H*D] float  (open_decoder.h:61)
+ */
+#ifndef FL_DECODE_ATTN_H
+#define FL_DECODE_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum fl_attn_status {
+    FL_ATTN_OK = 0,
+    FL_ATTN_ERR_NULL_POINTER = -1,  /* a required pointer is NULL */
+    FL_ATTN_ERR_HEAD_DIM = -2,      /* size_per_head not in {32,64,128,256,512,1024}
+                                       (reference: throw "invalid size_per_head!") */
+    FL_ATTN_ERR_SHAPE = -3,         /* non-positive B/H/L, or sizes beyond the grid limits */
+    FL_ATTN_ERR_POSITION = -4,      /* start_pos (+1) does not fit in total_len, bad rope_row */
+    FL_ATTN_ERR_WORKSPACE = -5,     /* workspace missing, too small or misaligned */
+    FL_ATTN_ERR_DTYPE = -6,         /* dtype is neither FL_ATTN_F32 nor FL_ATTN_F16 */
+    FL_ATTN_ERR_HIP = -7,           /* a HIP runtime call failed (see fl_attn_last_hip_error) */
+    FL_ATTN_ERR_ALIGNMENT = -8,     /* a tensor base is not 16-byte aligned */
+    FL_ATTN_ERR_ARGUMENT = -9       /* inconsistent optional arguments */
+} fl_attn_status;
+
+enum { FL_ATTN_F32 = 0, FL_ATTN_F16 = 1 };
+
+/* rope_row value meaning "rotate by the table row of each sequence's own position" */
+#define FL_ATTN_ROPE_AT_POSITION (-1)
+
+/* Problem shape; mirrors the OpenDecoder constructor arguments (open_decoder.h:66). */
+typedef struct fl_attn_desc {
+    int32_t batch_size;    /* B */
+    int32_t head_num;      /* H */
+    int32_t size_per_head; /* D */
+    int32_t total_len;     /* L = max_prompt_len + max_gen_len: rows per (b,h) in each cache */
+    int32_t dtype;         /* storage type of q/k_new/v_new and of both caches */
+    int32_t nsplit;        /* context splits per (b,h); 0 = chosen by the library */
+    float softmax_scale;   /* 0 = 1/sqrt(D) (open_decoder.cu:208) */
+    int32_t reserved;      /* must be 0 */
+} fl_attn_desc;
+
+/* Per-call operands; mirrors the arguments of OpenDecoder::forward (open_decoder.h:76-77). */
+typedef struct fl_attn_io {
+    const void *q;      /* [B,1,H,D] dtype; int32 accumulators when qkv_inp_scale != NULL */
+    const void *k_new;  /* same */
+    const void *v_new;  /* same */
+    void *k_cache;      /* [B,H,L,D] dtype; row start_pos is written, rows < start_pos are read */
+    void *v_cache;      /* same */
+    const float *freq_cis;            /* RoPE table */
+    const float *attn_mask;           /* NULL = no mask (decoder_kernels.cu:814) */
+    const int32_t *start_pos_per_seq; /* NULL, or [B] positions (ragged batches; an extension) */
+    float *out;                       /* [B, H*D]; may be NULL when out_int8 is given */
+    void *workspace;                  /* fl_decode_attn_workspace_bytes() bytes, 256-aligned */
+    size_t workspace_bytes;
+    int64_t mask_ld;       /* row stride of attn_mask in floats (the reference uses L) */
+    int32_t start_pos;     /* tokens already cached; the new token lands in row start_pos */
+    int32_t rope_row;      /* table row for RoPE, or FL_ATTN_ROPE_AT_POSITION */
+    int32_t max_start_pos; /* with start_pos_per_seq: upper bound of its entries, <0 = L-1 */
+    int32_t reserved;      /* must be 0 */
+    /* optional prologue: q/k_new/v_new are int32 [B,1,H,D]; x = acc*inp_scale[b]*w_scale[h*D+d] */
+    const float *qkv_inp_scale;  /* [B] or NULL */
+    const float *q_weight_scale; /* [H*D] */
+    const float *k_weight_scale; /* [H*D] */
+    const float *v_weight_scale; /* [H*D] */
+    /* optional epilogue: per-row absmax INT8 quantisation of out */
+    int8_t *out_int8; /* [B, H*D] or NULL */
+    float *out_scale; /* [B] (absmax/127), required with out_int8 */
+} fl_attn_io;
+
+/* Launch plan the library would use for a context of ctx rows (ctx = start_pos + 1). */
+typedef struct fl_attn_plan {
+    int32_t nsplit;       /* context splits per (b,h) */
+    int32_t chunk_rows;   /* cache rows per split */
+    int32_t threads;      /* threads per workgroup of the streaming kernel */
+    int32_t two_pass;     /* 1 when a combine pass follows the streaming pass */
+} fl_attn_plan;
+
+/* Bytes of scratch fl_decode_attn_forward needs for this shape (split partials; covers every
+ * start_pos < L).  Replaces the attention share of OpenDecoder::getWorkspaceSize
+ * (open_decoder.cu:54-67: query_out_buf_, key_out_buf_, value_out_fp_buf_, qk_buf_). */
+int fl_decode_attn_workspace_bytes(const fl_attn_desc *desc, size_t *bytes);
+
+/* The plan for a given context length (for logging and for the benchmark's byte accounting). */
+int fl_decode_attn_plan(const fl_attn_desc *desc, int32_t ctx, fl_attn_plan *plan);
+
+/* One decode step of attention for all (batch, head) pairs. */
+int fl_decode_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream);
+
+/* Same, restricted to some passes: bit 0 = streaming pass (RoPE, append, partial attention),
+ * bit 1 = combine pass (merge of split partials, optional INT8 epilogue).  Lets a profiler or
+ * benchmark time the bandwidth-bound kernel alone; fl_decode_attn_forward == passes 3. */
+int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream,
+                                  int passes);
+
+/* RoPE table producer on the device: rows x D floats, row r = [cos(r*w_0), sin(r*w_0), ...],
+ * w_i = base^(-2i/D).  Replaces launchPrecomputeFreqsCis (decoding_kernels.cu:85-135,
+ * called at decoding_sampling.cu:190) with correctly rounded sincos instead of fast intrinsics. */
+int fl_rope_table(float *freq_cis, int32_t rows, int32_t size_per_head, float base,
+                  void *hip_stream);
+
+/* Bytes of one layer's K (or V) cache, [B,H,L,D] in dtype: the per-layer stride a caller uses
+ * to carve its arena (decoding_sampling.cu:118-119, :180, :256-257). */
+int fl_kv_cache_bytes(const fl_attn_desc *desc, size_t *bytes);
+
+const char *fl_attn_strerror(int status);
+
+/* hipError_t of the most recent failing HIP call made by this library on this thread. */
+int fl_attn_last_hip_error(void);
+
+/* Library/ABI version: major*10000 + minor*100 + patch. */
+int fl_attn_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FL_DECODE_ATTN_H */
