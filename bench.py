@@ -1,0 +1,250 @@
+#!/usr/bin/env python3
+"""Decode-step self-attention benchmark (one MI355X).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3]
+
+One step = one pass of the hot path (RoPE -> KV append -> masked attention over the cache) for a
+whole batch, through the C ABI, on synthetic seeded inputs already resident in HBM.  Prints ONE
+JSON line.  `value` is algorithmic bytes per step / time per step (GB/s); `ms_per_step` carries the
+latency half of the metric.  `roofline` prices the streaming kernel alone (HIP events around
+back-to-back launches of that pass); `cpu_baseline` is the scalar CPU oracle timed on this
+machine's host cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E peak
+
+# name -> (B, H, D, ctx, L, dtype, extras)
+WORKLOADS = {
+    "cfg1": dict(B=1, H=4, D=64, ctx=128, L=128, dtype="f32", copies=64),
+    "cfg2": dict(B=8, H=32, D=128, ctx=1024, L=1024, dtype="f16", copies=6),
+    "cfg3": dict(B=64, H=32, D=128, ctx=2048, L=2048, dtype="f16", copies=1),
+    "cfg4": dict(B=1, H=32, D=128, ctx=4096, L=4096, dtype="f16", copies=12),
+    "cfg5": dict(B=32, H=40, D=128, ctx=None, L=4096, dtype="f16", copies=1, ragged=True),
+}
+HEADLINE = "cfg3"
+
+# HBM bytes per launch of the streaming kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
+# scaled by the factor the same counters read for a copy kernel of known size.  Filled in from
+# the summaries under profiles/ (None until measured for that workload).
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(B, H, D, e, sum_ctx, has_mask=False, mean_ctx=0):
+    """Bytes one step must move: K and V rows once, the token's q/k/v in, the two new rows out,
+    the fp32 output, one RoPE row (and one mask row when a mask is given)."""
+    kv = 2 * H * D * e * sum_ctx              # sum over sequences of ctx_b rows of K and of V
+    tok = 3 * B * H * D * e + 2 * B * H * D * e
+    out = B * H * D * 4
+    small = D * 4 + (int(mean_ctx) * 4 if has_mask else 0)
+    return kv + tok + out + small
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--nsplit", type=int, default=0, help="force the context split count (0 = library's choice)")
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="only run a plain 1 GiB -> 1 GiB elementwise copy kernel a few times (for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings), then exit")
+    ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path has no cross-GPU exchange); "
+              "run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from fasterllama_amd import capi, synth
+    from fasterllama_amd.decode_attn import DecodeAttention
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    capi.load()  # fails loudly when the HIP library is missing
+    dev = torch.device("cuda:0")
+    if args.calib_copy:
+        n = 1 << 28  # 2^28 floats = 1 GiB read + 1 GiB written per launch
+        src = torch.ones(n, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        print(json.dumps({"calib_copy": True, "bytes_read_per_launch": n * 4, "bytes_written_per_launch": n * 4,
+                          "launches": 5}), flush=True)
+        return 0
+    w = WORKLOADS[args.workload]
+    B, H, D, L = w["B"], w["H"], w["D"], w["L"]
+    np_dt = np.float16 if w["dtype"] == "f16" else np.float32
+    t_dt = torch.float16 if w["dtype"] == "f16" else torch.float32
+    e = 2 if w["dtype"] == "f16" else 4
+    ragged = bool(w.get("ragged"))
+    copies = w["copies"]
+
+    if ragged:
+        lens = synth.uniform_int(B, 1, L, synth.TENSOR_LENS, args.seed)
+        pos_h = (lens - 1).astype(np.int32)
+        sum_ctx, max_ctx = int(lens.sum()), int(lens.max())
+    else:
+        lens = np.full(B, w["ctx"], np.int32)
+        pos_h = None
+        sum_ctx, max_ctx = B * w["ctx"], w["ctx"]
+    start_pos = max_ctx - 1
+
+    # ---- inputs: generated on the host by the seeded generator, then copied to HBM once
+    t0 = time.time()
+    q_h = synth.normal((B, 1, H, D), np_dt, synth.TENSOR_Q, args.seed)
+    k_h = synth.normal((B, 1, H, D), np_dt, synth.TENSOR_K_NEW, args.seed)
+    v_h = synth.normal((B, 1, H, D), np_dt, synth.TENSOR_V_NEW, args.seed)
+    kc_h = synth.normal((B, H, L, D), np_dt, synth.TENSOR_K_CACHE, args.seed)
+    vc_h = synth.normal((B, H, L, D), np_dt, synth.TENSOR_V_CACHE, args.seed)
+    if ragged:  # rows the step must never read
+        for b in range(B):
+            kc_h[b, :, lens[b]:, :] = np.nan
+            vc_h[b, :, lens[b]:, :] = np.nan
+    freq_h = synth.freq_cis_table(L, D)
+    q, k, v = (torch.from_numpy(a).to(dev) for a in (q_h, k_h, v_h))
+    freq = torch.from_numpy(freq_h).to(dev)
+    pos_d = torch.from_numpy(pos_h).to(dev) if ragged else None
+    # small workloads rotate over several cache copies so the rows do not sit in the 256 MB MALL
+    caches = []
+    for c in range(copies):
+        caches.append((torch.from_numpy(kc_h).to(dev), torch.from_numpy(vc_h).to(dev)))
+    out = torch.empty(B, H * D, dtype=torch.float32, device=dev)
+    torch.cuda.synchronize()
+    gen_s = time.time() - t0
+
+    op = DecodeAttention(B, H, D, L, t_dt, nsplit=args.nsplit, device=dev)
+    plan = op.plan(max_ctx)
+    ios = [op.make_io(q, k, v, kc, vc, freq, out, start_pos=start_pos, start_pos_per_seq=pos_d,
+                      max_start_pos=start_pos if ragged else -1) for kc, vc in caches]
+    stream = torch.cuda.current_stream(dev)
+
+    def run(n, passes=3):
+        for i in range(n):
+            st = op.launch(ios[i % copies], passes=passes, stream=stream)
+            if st != 0:
+                raise capi.FlAttnError(st, capi.strerror(st))
+
+    # ---- timed region: W warm-up steps, then exactly K steps between two events on the stream
+    run(args.warmup)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    h0 = time.perf_counter()
+    ev0.record(stream)
+    run(args.steps)
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    host_ms = (time.perf_counter() - h0) * 1e3
+    step_ms = ev0.elapsed_time(ev1) / args.steps
+    out_gpu = out.cpu().numpy().copy()
+
+    # ---- the streaming kernel alone (pass 1), same launches, same stream
+    run(max(3, args.warmup // 4), passes=1)
+    torch.cuda.synchronize()
+    ev2, ev3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev2.record(stream)
+    run(args.steps, passes=1)
+    ev3.record(stream)
+    torch.cuda.synchronize()
+    kern_ms = ev2.elapsed_time(ev3) / args.steps
+
+    alg = algorithmic_bytes(B, H, D, e, sum_ctx)
+    gbps = alg / (step_ms * 1e-3) / 1e9
+    kern_gbps = alg / (kern_ms * 1e-3) / 1e9
+
+    # ---- CPU baseline: the scalar oracle on a bounded sample of the same inputs (~10-20 s of CPU work)
+    cpu = None
+    max_err = None
+    if not args.no_cpu:
+        from oracle import ref  # checker / baseline only
+        per_seq = 2 * H * D * e * (sum_ctx / B)
+        ns = args.cpu_seqs or max(1, min(B, int(round(0.5e9 / per_seq))))  # ~0.5 GB of K+V per pass
+        sl = slice(0, ns)
+        pos_s = pos_h[sl] if ragged else None
+        sample_bytes = algorithmic_bytes(ns, H, D, e, int(lens[sl].sum()))
+
+        def cpu_leg(threads, budget_s, max_reps):
+            kc_s, vc_s = kc_h[sl].copy(), vc_h[sl].copy()
+            times, res = [], None
+            while sum(times) < budget_s and len(times) < max_reps:
+                t1 = time.perf_counter()
+                res = ref.decode_attn(q_h[sl], k_h[sl], v_h[sl], kc_s, vc_s, freq_h, start_pos=start_pos,
+                                      start_pos_per_seq=pos_s, threads=threads)
+                times.append(time.perf_counter() - t1)
+            return res, min(times), len(times), sum(times)
+
+        out_ref, cpu_1t, reps_1t, total_1t = cpu_leg(1, 10.0, 50)
+        nthreads = max(1, min(16, os.cpu_count() or 1))
+        _, cpu_nt, reps_nt, total_nt = cpu_leg(nthreads, 4.0, 50)
+        max_err = float(np.abs(out_gpu[sl] - out_ref).max())
+        cpu = {
+            "value": round(sample_bytes / cpu_1t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"first {ns} of {B} sequences of the same seeded inputs ({sample_bytes / 1e6:.0f} MB "
+                      f"algorithmic per pass), scalar oracle, 1 thread, best of {reps_1t} passes "
+                      f"({total_1t:.1f} s of CPU work)",
+            "us_per_step_scaled_to_full_batch": round(cpu_1t * B / ns * 1e6, 1),
+            "openmp": {"value": round(sample_bytes / cpu_nt / 1e9, 4), "unit": "GB/s", "cores": nthreads,
+                       "passes": reps_nt, "us_per_step_scaled_to_full_batch": round(cpu_nt * B / ns * 1e6, 1)},
+            "gpu_vs_oracle_max_abs_err": max_err,
+        }
+
+    line = {
+        "metric": "decode-attn us/step + HBM GB/s (% peak), LLaMA2-7B heads b=64 ctx=2048 fp16"
+                  if args.workload == HEADLINE else f"decode-attn us/step + HBM GB/s (% peak), {args.workload}",
+        "value": round(gbps, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_ms, 6),
+        "us_per_step": round(step_ms * 1e3, 2),
+        "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 storage / f32 accumulate" if w["dtype"] == "f16" else "f32",
+        "data": "synthetic (seeded splitmix64 + Box-Muller N(0,1), seed %d)" % args.seed,
+        "config": {
+            "workload": f"{args.workload}: decode self-attention step, B={B} H={H} D={D} "
+                        + (f"ragged ctx U[1,{L}] (sum {sum_ctx})" if ragged else f"ctx={max_ctx}")
+                        + f" L={L} {w['dtype']} KV cache, RoPE at position, no mask",
+            "batch": B, "heads": H, "head_dim": D, "ctx": max_ctx if not ragged else None,
+            "sum_ctx": sum_ctx, "cache_rows": L, "cache_copies_rotated": copies,
+            "nsplit": plan.nsplit, "chunk_rows": plan.chunk_rows, "two_pass": bool(plan.two_pass),
+            "algorithmic_bytes_per_step": alg,
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": round(kern_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(kern_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "kernel": "decode_attn_split_kernel", "kernel_us": round(kern_ms * 1e3, 2),
+        },
+        "cpu_baseline": cpu,
+        "host_ms_total": round(host_ms, 3),
+        "input_gen_s": round(gen_s, 2),
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
