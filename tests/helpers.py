@@ -60,7 +60,7 @@ class Case:
         f, m, pos = d(self.freq), d(self.mask), d(self.pos)
         out = op.forward(q, k, v, kc, vc, f, start_pos=self.start_pos, rope_row=self.rope_row,
                          attn_mask=m, start_pos_per_seq=pos,
-                         max_start_pos=int(self.pos.max()) if self.pos is not None else -1)
+                         max_start_pos=min(int(self.pos.max()), self.L - 1) if self.pos is not None else -1)
         torch.cuda.synchronize(device)
         return out.cpu().numpy(), kc.cpu().numpy(), vc.cpu().numpy(), op
 
