@@ -1,0 +1,266 @@
+// Drop-in check of the C++ OpenDecoder mirror on a real GPU: the calls a FasterLLaMA caller makes
+// (constructor, getWorkspaceSize, initialize, forward) plus decodeAttention, compared with the CPU
+// oracle (linked from oracle/libfl_ref.so — checker only).  Prints one line per check and exits
+// non-zero on the first failure.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <stdexcept>
+#include <vector>
+
+#include "open_decoder.h"
+
+extern "C" {
+int fl_ref_decode_attn(int dtype, int B, int H, int D, int L, const void *q, const void *k_new, const void *v_new,
+                       void *k_cache, void *v_cache, const float *freq_cis, int rope_row, const float *attn_mask,
+                       int64_t mask_ld, int start_pos, const int32_t *start_pos_per_seq, float scale, float *out,
+                       int acc_double, int threads);
+int fl_ref_decode_attn_i32(int dtype, int B, int H, int D, int L, const int32_t *q_acc, const int32_t *k_acc,
+                           const int32_t *v_acc, const float *inp_scale, const float *wq_scale, const float *wk_scale,
+                           const float *wv_scale, void *k_cache, void *v_cache, const float *freq_cis, int rope_row,
+                           const float *attn_mask, int64_t mask_ld, int start_pos, const int32_t *start_pos_per_seq,
+                           float scale, float *out, int acc_double, int threads);
+int fl_ref_attn_quantize(int B, int HD, const float *attn, int8_t *out_q, float *out_scale);
+int fl_ref_freq_cis(float *table, int rows, int D, double base);
+uint16_t fl_ref_float_to_half(float f);
+}
+
+using namespace FasterLLaMA;
+
+#define HIP_OK(x)                                                                                  \
+    do {                                                                                           \
+        hipError_t e_ = (x);                                                                       \
+        if (e_ != hipSuccess) {                                                                    \
+            std::printf("FAIL hip error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+            std::exit(2);                                                                          \
+        }                                                                                          \
+    } while (0)
+
+static uint64_t g_state = 0x1234567ull;
+static float frand() // uniform in [-1, 1)
+{
+    g_state = g_state * 6364136223846793005ull + 1442695040888963407ull;
+    return (float)((g_state >> 40) & 0xFFFFFF) / 8388608.0f - 1.0f;
+}
+
+template <typename T> struct DevBuf {
+    T *p = nullptr;
+    size_t n = 0;
+    explicit DevBuf(size_t n_) : n(n_) { HIP_OK(hipMalloc(&p, n * sizeof(T))); }
+    ~DevBuf() { (void)hipFree(p); }
+    void up(const void *h) { HIP_OK(hipMemcpy(p, h, n * sizeof(T), hipMemcpyHostToDevice)); }
+    void down(void *h) const { HIP_OK(hipMemcpy(h, p, n * sizeof(T), hipMemcpyDeviceToHost)); }
+};
+
+static int g_fail = 0;
+static void report(const char *name, bool ok, double detail = 0.0)
+{
+    std::printf("%s %s (%.3e)\n", ok ? "PASS" : "FAIL", name, detail);
+    std::fflush(stdout);
+    if (!ok) g_fail = 1;
+}
+
+struct HookCtx {
+    const int32_t *q, *k, *v;
+    const float *scale;
+    int8_t *seen_int8;
+    float *seen_scale;
+    size_t hidden;
+    int calls_pre = 0, calls_post = 0;
+};
+
+template <typename T>
+static void qkvHook(void *user, const T *, int32_t *qb, int32_t *kb, int32_t *vb, float *sb, int B, hipStream_t s)
+{
+    HookCtx *c = static_cast<HookCtx *>(user);
+    const size_t bytes = (size_t)B * c->hidden * sizeof(int32_t);
+    HIP_OK(hipMemcpyAsync(qb, c->q, bytes, hipMemcpyDeviceToDevice, s));
+    HIP_OK(hipMemcpyAsync(kb, c->k, bytes, hipMemcpyDeviceToDevice, s));
+    HIP_OK(hipMemcpyAsync(vb, c->v, bytes, hipMemcpyDeviceToDevice, s));
+    HIP_OK(hipMemcpyAsync(sb, c->scale, (size_t)B * sizeof(float), hipMemcpyDeviceToDevice, s));
+    c->calls_pre++;
+}
+
+template <typename T>
+static void postHook(void *user, const int8_t *a8, const float *as, const T *, T *, int B, hipStream_t s)
+{
+    HookCtx *c = static_cast<HookCtx *>(user);
+    HIP_OK(hipMemcpyAsync(c->seen_int8, a8, (size_t)B * c->hidden, hipMemcpyDeviceToDevice, s));
+    HIP_OK(hipMemcpyAsync(c->seen_scale, as, (size_t)B * sizeof(float), hipMemcpyDeviceToDevice, s));
+    c->calls_post++;
+}
+
+template <typename CacheT> static CacheT toCache(float x);
+template <> float toCache<float>(float x) { return x; }
+template <> __half toCache<__half>(float x)
+{
+    uint16_t b = fl_ref_float_to_half(x);
+    __half h;
+    std::memcpy(&h, &b, 2);
+    return h;
+}
+
+template <OperationType Op, typename CacheT> static void runAll(const char *tag)
+{
+    typedef typename DecoderTransformerTraits<Op>::DataType DataT;
+    const int B = 3, H = 8, D = 128, prompt = 40, gen = 24, L = prompt + gen, P = 50, HD = H * D;
+    const int code = std::is_same<CacheT, float>::value ? 0 : 1;
+    char name[128];
+
+    std::vector<float> freq((size_t)L * D), mask((size_t)L * L);
+    fl_ref_freq_cis(freq.data(), L, D, 10000.0);
+    for (int r = 0; r < L; ++r)
+        for (int c = 0; c < L; ++c) mask[(size_t)r * L + c] = c > r ? -1e5f : 0.0f; // causal (samples/test.cu:427-437)
+
+    std::vector<CacheT> q((size_t)B * HD), k(q.size()), v(q.size()), kc((size_t)B * H * L * D), vc(kc.size());
+    for (auto &x : q) x = toCache<CacheT>(frand());
+    for (auto &x : k) x = toCache<CacheT>(frand());
+    for (auto &x : v) x = toCache<CacheT>(frand());
+    for (auto &x : kc) x = toCache<CacheT>(frand());
+    for (auto &x : vc) x = toCache<CacheT>(frand());
+
+    DevBuf<float> d_freq(freq.size()), d_mask(mask.size()), d_out((size_t)B * HD);
+    DevBuf<CacheT> d_q(q.size()), d_k(k.size()), d_v(v.size()), d_kc(kc.size()), d_vc(vc.size());
+    d_freq.up(freq.data()); d_mask.up(mask.data());
+    d_q.up(q.data()); d_k.up(k.data()); d_v.up(v.data()); d_kc.up(kc.data()); d_vc.up(vc.data());
+
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+
+    OpenDecoder<Op, OperationType::INT8> dec(B, prompt, gen, H, D, 4 * HD);
+    const int ws_bytes = dec.getWorkspaceSize();
+    DevBuf<char> d_ws((size_t)ws_bytes);
+    DecoderInitParam<DataT, int8_t> param;
+    param.attn_mask = d_mask.p;
+    param.stream = stream;
+
+    std::vector<float> wq(HD), wk(HD), wv(HD), s_in(B);
+    for (auto &x : wq) x = 0.01f + 0.01f * (frand() + 1.0f);
+    for (auto &x : wk) x = 0.01f + 0.01f * (frand() + 1.0f);
+    for (auto &x : wv) x = 0.01f + 0.01f * (frand() + 1.0f);
+    for (auto &x : s_in) x = 0.002f + 0.001f * (frand() + 1.0f);
+    DevBuf<float> d_wq(HD), d_wk(HD), d_wv(HD), d_sin(B);
+    d_wq.up(wq.data()); d_wk.up(wk.data()); d_wv.up(wv.data()); d_sin.up(s_in.data());
+    param.attention.query_weight.weight_scale = d_wq.p;
+    param.attention.key_weight.weight_scale = d_wk.p;
+    param.attention.value_weight.weight_scale = d_wv.p;
+    dec.initialize(param, d_ws.p);
+
+    // ---- 1. decodeAttention on float/half operands vs the oracle
+    {
+        std::vector<CacheT> kc_ref(kc), vc_ref(vc), kc_got(kc.size()), vc_got(vc.size());
+        std::vector<float> want((size_t)B * HD), got(want.size());
+        fl_ref_decode_attn(code, B, H, D, L, q.data(), k.data(), v.data(), kc_ref.data(), vc_ref.data(), freq.data(), -1,
+                           mask.data(), L, P, nullptr, 1.0f / std::sqrt((float)D), want.data(), 1, 1);
+        dec.decodeAttention(d_q.p, d_k.p, d_v.p, d_freq.p, d_kc.p, d_vc.p, d_out.p, P);
+        HIP_OK(hipStreamSynchronize(stream));
+        d_out.down(got.data()); d_kc.down(kc_got.data()); d_vc.down(vc_got.data());
+        double worst = 0, scale = 0;
+        for (float w : want) scale = std::fmax(scale, std::fabs(w));
+        for (size_t i = 0; i < want.size(); ++i) {
+            double tol = code ? 2e-3 : 1e-5 * std::fmax(std::fabs(want[i]), scale);
+            worst = std::fmax(worst, std::fabs((double)got[i] - want[i]) / tol);
+        }
+        std::snprintf(name, sizeof name, "%s decodeAttention output", tag);
+        report(name, worst <= 1.0, worst);
+        std::snprintf(name, sizeof name, "%s decodeAttention caches bit-exact", tag);
+        report(name, !std::memcmp(kc_got.data(), kc_ref.data(), kc.size() * sizeof(CacheT)) &&
+                         !std::memcmp(vc_got.data(), vc_ref.data(), vc.size() * sizeof(CacheT)));
+    }
+
+    // ---- 2. forward() with external stages: int32 accumulators in, INT8 + scale out
+    std::vector<int32_t> qi((size_t)B * HD), ki(qi.size()), vi(qi.size());
+    for (auto &x : qi) x = (int32_t)(frand() * 20000.f);
+    for (auto &x : ki) x = (int32_t)(frand() * 20000.f);
+    for (auto &x : vi) x = (int32_t)(frand() * 20000.f);
+    DevBuf<int32_t> d_qi(qi.size()), d_ki(ki.size()), d_vi(vi.size());
+    d_qi.up(qi.data()); d_ki.up(ki.data()); d_vi.up(vi.data());
+    DevBuf<int8_t> d_seen8((size_t)B * HD);
+    DevBuf<float> d_seens(B);
+    HookCtx ctx{d_qi.p, d_ki.p, d_vi.p, d_sin.p, d_seen8.p, d_seens.p, (size_t)HD};
+    {
+        d_kc.up(kc.data()); d_vc.up(vc.data());
+        DecoderExternalStages<DataT> stages;
+        stages.user = &ctx;
+        stages.qkv_projection = qkvHook<DataT>;
+        stages.post_attention = postHook<DataT>;
+        dec.setExternalStages(stages);
+        DevBuf<DataT> d_from((size_t)B * HD), d_dec_out((size_t)B * HD);
+        dec.forward(d_from.p, d_freq.p, d_kc.p, d_vc.p, d_dec_out.p, P, 1);
+        HIP_OK(hipStreamSynchronize(stream));
+
+        std::vector<CacheT> kc_ref(kc), vc_ref(vc), kc_got(kc.size());
+        std::vector<float> want((size_t)B * HD), want_s(B), got_s(B);
+        std::vector<int8_t> want8((size_t)B * HD), got8(want8.size());
+        fl_ref_decode_attn_i32(code, B, H, D, L, qi.data(), ki.data(), vi.data(), s_in.data(), wq.data(), wk.data(), wv.data(),
+                               kc_ref.data(), vc_ref.data(), freq.data(), -1, mask.data(), L, P, nullptr,
+                               1.0f / std::sqrt((float)D), want.data(), 1, 1);
+        fl_ref_attn_quantize(B, HD, want.data(), want8.data(), want_s.data());
+        d_seen8.down(got8.data()); d_seens.down(got_s.data()); d_kc.down(kc_got.data());
+        int worst8 = 0;
+        for (size_t i = 0; i < want8.size(); ++i) worst8 = std::max(worst8, std::abs((int)got8[i] - (int)want8[i]));
+        double worst_s = 0;
+        for (int b = 0; b < B; ++b) worst_s = std::fmax(worst_s, std::fabs(got_s[b] - want_s[b]) / want_s[b]);
+        std::snprintf(name, sizeof name, "%s forward int8 within one step", tag);
+        report(name, worst8 <= 1 && ctx.calls_pre == 1 && ctx.calls_post == 1, worst8);
+        std::snprintf(name, sizeof name, "%s forward output scale", tag);
+        report(name, worst_s <= 1e-5, worst_s);
+        std::snprintf(name, sizeof name, "%s forward k_cache bit-exact", tag);
+        report(name, !std::memcmp(kc_got.data(), kc_ref.data(), kc.size() * sizeof(CacheT)));
+    }
+
+    // ---- 3. literal RoPE row: the appended key equals the unrotated key (row 0 = identity)
+    {
+        d_kc.up(kc.data()); d_vc.up(vc.data());
+        dec.setLiteralRopeRow(true);
+        dec.decodeAttention(d_q.p, d_k.p, d_v.p, d_freq.p, d_kc.p, d_vc.p, d_out.p, P);
+        HIP_OK(hipStreamSynchronize(stream));
+        dec.setLiteralRopeRow(false);
+        std::vector<CacheT> kc_got(kc.size());
+        d_kc.down(kc_got.data());
+        bool same = true;
+        for (int b = 0; b < B && same; ++b)
+            for (int h = 0; h < H && same; ++h)
+                same = !std::memcmp(&kc_got[(((size_t)b * H + h) * L + P) * D], &k[((size_t)b * H + h) * D], D * sizeof(CacheT));
+        std::snprintf(name, sizeof name, "%s literal RoPE row stores k unrotated", tag);
+        report(name, same);
+    }
+
+    // ---- 4. error behaviour: std::runtime_error, never exit()
+    {
+        DevBuf<DataT> d_from((size_t)B * HD), d_dec_out((size_t)B * HD);
+        int caught = 0;
+        try { dec.forward(d_from.p, d_freq.p, d_kc.p, d_vc.p, d_dec_out.p, 0, 2); } catch (std::runtime_error &) { caught++; }
+        try { dec.forward(d_from.p, d_freq.p, d_kc.p, d_vc.p, d_dec_out.p, L, 1); } catch (std::runtime_error &) { caught++; }
+        try { dec.decodeAttention(d_q.p, d_k.p, d_v.p, (const float *)nullptr, d_kc.p, d_vc.p, d_out.p, P); } catch (std::runtime_error &) { caught++; }
+        try {
+            OpenDecoder<Op, OperationType::INT8> bad(B, prompt, gen, H, 96, 4 * HD); // reference: throw "invalid size_per_head!"
+            (void)bad.getWorkspaceSize();
+        } catch (std::runtime_error &) { caught++; }
+        try {
+            OpenDecoder<Op, OperationType::INT8> fresh(B, prompt, gen, H, D, 4 * HD); // no stages installed
+            fresh.initialize(param, d_ws.p);
+            fresh.forward(d_from.p, d_freq.p, d_kc.p, d_vc.p, d_dec_out.p, P, 1);
+        } catch (std::runtime_error &) { caught++; }
+        std::snprintf(name, sizeof name, "%s errors surface as std::runtime_error", tag);
+        report(name, caught == 5, caught);
+    }
+    HIP_OK(hipStreamDestroy(stream));
+}
+
+int main()
+{
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n < 1) {
+        std::printf("FAIL no GPU\n");
+        return 3;
+    }
+    runAll<OperationType::FP32, float>("OpenDecoder<FP32,INT8>/float-cache");
+    runAll<OperationType::FP16, float>("OpenDecoder<FP16,INT8>/float-cache");
+    runAll<OperationType::FP16, __half>("OpenDecoder<FP16,INT8>/half-cache");
+    std::printf(g_fail ? "SOME CHECKS FAILED\n" : "ALL CHECKS PASSED\n");
+    return g_fail;
+}
