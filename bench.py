@@ -31,6 +31,9 @@ WORKLOADS = {
     "cfg3": dict(B=64, H=32, D=128, ctx=2048, L=2048, dtype="f16", copies=1),
     "cfg4": dict(B=1, H=32, D=128, ctx=4096, L=4096, dtype="f16", copies=12),
     "cfg5": dict(B=32, H=40, D=128, ctx=None, L=4096, dtype="f16", copies=1, ragged=True),
+    # exploration shapes (not BASELINE configurations)
+    "x13b_uniform": dict(B=32, H=40, D=128, ctx=4096, L=4096, dtype="f16", copies=1),
+    "x7b_halffull": dict(B=64, H=32, D=128, ctx=2048, L=4096, dtype="f16", copies=1),
 }
 HEADLINE = "cfg3"
 
@@ -133,7 +136,7 @@ def main() -> int:
     gen_s = time.time() - t0
 
     op = DecodeAttention(B, H, D, L, t_dt, nsplit=args.nsplit, device=dev)
-    plan = op.plan(max_ctx)
+    plan = op.plan(max_ctx, ragged)
     ios = [op.make_io(q, k, v, kc, vc, freq, out, start_pos=start_pos, start_pos_per_seq=pos_d,
                       max_start_pos=start_pos if ragged else -1) for kc, vc in caches]
     stream = torch.cuda.current_stream(dev)

@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "lib", "libfl_decode_attn.so")
+# FL_DECODE_ATTN_LIB points at another build of the same library (kernel tuning experiments)
+LIB_PATH = os.environ.get("FL_DECODE_ATTN_LIB") or os.path.join(_PKG, "lib", "libfl_decode_attn.so")
 
 FL_ATTN_F32 = 0
 FL_ATTN_F16 = 1
@@ -112,7 +113,7 @@ def load() -> C.CDLL:
     lib.fl_decode_attn_workspace_bytes.restype = C.c_int
     lib.fl_kv_cache_bytes.argtypes = [C.POINTER(AttnDesc), C.POINTER(C.c_size_t)]
     lib.fl_kv_cache_bytes.restype = C.c_int
-    lib.fl_decode_attn_plan.argtypes = [C.POINTER(AttnDesc), C.c_int32, C.POINTER(AttnPlan)]
+    lib.fl_decode_attn_plan.argtypes = [C.POINTER(AttnDesc), C.c_int32, C.c_int32, C.POINTER(AttnPlan)]
     lib.fl_decode_attn_plan.restype = C.c_int
     lib.fl_decode_attn_forward.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnIO), C.c_void_p]
     lib.fl_decode_attn_forward.restype = C.c_int

@@ -6,7 +6,10 @@
 // (:858-884), cache append (:597-632), Q K^T GEMV, block softmax (:800-835) and P V GEMV.
 //
 // Work decomposition
-//   grid = (nsplit, H, B); one workgroup streams `chunk` consecutive cache rows of one (b, h).
+//   grid = nsplit * B * H workgroups, linear id = split * (B*H) + (b*H + h); one workgroup streams
+//   `chunk` consecutive cache rows of one (b, h).  Consecutive ids go round-robin to the 8 XCDs, so
+//   with (b,h) fastest every XCD receives the same mix of splits: in a ragged batch the high splits
+//   are empty for short sequences, and a split-fastest order would starve the XCDs that own them.
 //   A row of D elements is 16-byte chunks; LPR = min(64, D*sizeof(T)/16) lanes own one row, so a
 //   wave covers 64/LPR rows per load instruction and every load instruction of a workgroup
 //   touches one contiguous span of the cache.  Each lane-group keeps a private online-softmax
@@ -17,6 +20,12 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
+
+// Every fused multiply-add in this file is written as fmaf(); the compiler must not form others,
+// so that e.g. a zero mask row and a NULL mask give bit-identical outputs.
+#pragma clang fp contract(off)
 
 namespace flattn {
 
@@ -31,14 +40,13 @@ struct Params {
     float *part_m; // [B*H, split_cap]
     float *part_l; // [B*H, split_cap]
     const float *inp_scale, *wq_scale, *wk_scale, *wv_scale;
-    int8_t *out_int8;
-    float *out_scale;
     int64_t mask_ld;
     int32_t B, H, L;
     int32_t start_pos, rope_row;
     int32_t chunk;     // cache rows per split
     int32_t split_cap; // stride of the partial arrays along the split axis
     int32_t direct;    // 1: single split, write normalised output straight to `out`
+    int32_t log2_domain; // 1: partial maxima are in base-2 units (fast-exp streaming kernel)
     float scale;
 };
 
@@ -65,6 +73,35 @@ __device__ __forceinline__ float group_sum(float x)
     if constexpr (LPR >= 64) x += __shfl_xor(x, 32);
     return x;
 }
+
+// Same reduction for N independent values, one butterfly step at a time across all of them, so
+// the data-parallel-primitive wait states of one value are filled by the others.
+template <int LPR, int N>
+__device__ __forceinline__ void group_sum_n(float (&x)[N])
+{
+#define FLATTN_STEP(COND, EXPR)                     \
+    if constexpr (COND) {                           \
+        _Pragma("unroll") for (int u = 0; u < N; ++u) x[u] += (EXPR); \
+    }
+    FLATTN_STEP(LPR >= 2, dpp_move<0xB1>(x[u]))
+    FLATTN_STEP(LPR >= 4, dpp_move<0x4E>(x[u]))
+    FLATTN_STEP(LPR >= 8, dpp_move<0x141>(x[u]))
+    FLATTN_STEP(LPR >= 16, dpp_move<0x140>(x[u]))
+    FLATTN_STEP(LPR >= 32, __shfl_xor(x[u], 16))
+    FLATTN_STEP(LPR >= 64, __shfl_xor(x[u], 32))
+#undef FLATTN_STEP
+}
+
+// exp in the softmax.  Natural domain: expf, as the reference (decoder_kernels.cu:824).
+// Base-2 domain (FAST): scores are pre-multiplied by log2(e) and one v_exp_f32 evaluates 2^x.
+template <bool FAST>
+__device__ __forceinline__ float softmax_exp(float x)
+{
+    if constexpr (FAST) return __builtin_amdgcn_exp2f(x);
+    else return expf(x);
+}
+
+constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ float wave_max(float x)
 {
@@ -138,8 +175,25 @@ __device__ __forceinline__ void load_token_chunk(const void *base, size_t elem_o
 
 // ---------------------------------------------------------------- streaming (split) kernel
 
-template <typename T, int D, int WAVES, int UNROLL>
-__global__ __launch_bounds__(WAVES * 64) void decode_attn_split_kernel(const Params p)
+#ifndef FLATTN_MIN_WAVES_PER_EU
+#define FLATTN_MIN_WAVES_PER_EU 8
+#endif
+
+// Occupancy the register allocator must leave room for: 8 waves per SIMD (<= 64 VGPRs) when one
+// lane owns a single 16-byte chunk of the row, fewer for the large head sizes.
+template <typename T, int D>
+constexpr int min_waves_per_eu()
+{
+    constexpr int cpl = (D / Vec16<T>::N) <= 64 ? 1 : (D / Vec16<T>::N) / 64;
+    if (D * (int)sizeof(T) < 128) return 4; // 16 rows per wave: the group merge needs the registers
+    return cpl == 1 ? FLATTN_MIN_WAVES_PER_EU : (cpl == 2 ? 4 : 2);
+}
+
+// FAST selects the base-2 softmax (fp16 storage); the fp32-storage kernels keep expf.
+template <typename T, int D, int WAVES, int UNROLL, bool HAS_MASK, bool FAST>
+__global__ __launch_bounds__(WAVES * 64)
+__attribute__((amdgpu_waves_per_eu(min_waves_per_eu<T, D>(), 8)))
+void decode_attn_split_kernel(const Params p)
 {
     typedef typename Vec16<T>::type V;
     constexpr int VEC = Vec16<T>::N;
@@ -149,15 +203,17 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attn_split_kernel(const Par
     constexpr int GPW = 64 / LPR;           // rows per wave per load instruction
     constexpr int GROUPS = WAVES * GPW;     // rows per workgroup per load instruction
     constexpr int EPL = CPL * VEC;          // elements of a row owned by one lane
+    constexpr int ROW_BYTES = D * (int)sizeof(T);
     static_assert(CH * VEC == D && LPR * CPL == CH, "head size must tile into 16-byte chunks");
 
     __shared__ float s_o[GROUPS][D];
     __shared__ float s_m[GROUPS];
     __shared__ float s_l[GROUPS];
 
-    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int H = p.H, L = p.L;
-    const int bh = b * H + h;
+    const int BH = p.B * H;
+    const int split = blockIdx.x / BH, bh = blockIdx.x % BH;
+    const int b = bh / H, h = bh % H;
     const int P = p.pos_per_seq ? p.pos_per_seq[b] : p.start_pos;
     const int tid = threadIdx.x;
 
@@ -198,12 +254,17 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attn_split_kernel(const Par
         }
     }
 
-    const T *Kb = reinterpret_cast<const T *>(p.k_cache) + (size_t)bh * L * D;
-    const T *Vb = reinterpret_cast<const T *>(p.v_cache) + (size_t)bh * L * D;
-    const float *mrow = p.attn_mask ? p.attn_mask + (size_t)P * p.mask_ld : nullptr;
-    const float scale = p.scale;
+    // Uniform (scalar) base of this (b,h) plus a 32-bit per-lane byte offset: the loads below are
+    // "scalar base + vector offset" with no per-row 64-bit vector address arithmetic.
+    const char *Kb = reinterpret_cast<const char *>(p.k_cache) + (size_t)bh * L * ROW_BYTES;
+    const char *Vb = reinterpret_cast<const char *>(p.v_cache) + (size_t)bh * L * ROW_BYTES;
+    const uint32_t lane_off = (uint32_t)(group * ROW_BYTES + lig * 16);
+    const float *mrow = HAS_MASK ? p.attn_mask + (size_t)P * p.mask_ld : nullptr;
+    // v = qk*scaler + mask (decoder_kernels.cu:815); the base-2 path folds log2(e) into both terms
+    const float scale = FAST ? p.scale * kLog2e : p.scale;
+    const float floor_m = FAST ? kMaxFloor * kLog2e : kMaxFloor;
 
-    float m = kMaxFloor, l = 0.f;
+    float m = floor_m, l = 0.f;
     float o[EPL];
 #pragma unroll
     for (int e = 0; e < EPL; ++e) o[e] = 0.f;
@@ -214,28 +275,32 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attn_split_kernel(const Par
         V kv[UNROLL][CPL], vv[UNROLL][CPL];
         float mk[UNROLL];
         bool ok[UNROLL];
+        const char *kt = Kb + (size_t)r0 * ROW_BYTES; // uniform
+        const char *vt = Vb + (size_t)r0 * ROW_BYTES;
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            int row = r0 + u * GROUPS + group;
-            ok[u] = !CHECK || row < cache_end;
-            if (CHECK && !ok[u]) row = r0; // any valid row; its data is discarded
-            const T *kp = Kb + (size_t)row * D + lig * VEC;
+            uint32_t off = lane_off + (uint32_t)(u * GROUPS * ROW_BYTES);
+            ok[u] = !CHECK || (r0 + u * GROUPS + group) < cache_end;
+            if (CHECK && !ok[u]) off = (uint32_t)(lig * 16); // row r0: valid; its data is discarded
 #pragma unroll
             for (int c = 0; c < CPL; ++c)
-                kv[u][c] = __builtin_nontemporal_load(reinterpret_cast<const V *>(kp + c * LPR * VEC));
-            mk[u] = mrow ? mrow[row] : 0.f;
+                kv[u][c] = __builtin_nontemporal_load(reinterpret_cast<const V *>(kt + off + c * LPR * 16));
+            if constexpr (HAS_MASK) {
+                const int row = (CHECK && !ok[u]) ? r0 : r0 + u * GROUPS + group;
+                mk[u] = mrow[row];
+            } else {
+                mk[u] = 0.f;
+            }
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            int row = r0 + u * GROUPS + group;
-            if (CHECK && !ok[u]) row = r0;
-            const T *vp = Vb + (size_t)row * D + lig * VEC;
+            uint32_t off = lane_off + (uint32_t)(u * GROUPS * ROW_BYTES);
+            if (CHECK && !ok[u]) off = (uint32_t)(lig * 16);
 #pragma unroll
             for (int c = 0; c < CPL; ++c)
-                vv[u][c] = __builtin_nontemporal_load(reinterpret_cast<const V *>(vp + c * LPR * VEC));
+                vv[u][c] = __builtin_nontemporal_load(reinterpret_cast<const V *>(vt + off + c * LPR * 16));
         }
         float s[UNROLL];
-        float tmax = m;
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             float acc = 0.f;
@@ -243,12 +308,17 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attn_split_kernel(const Par
             for (int c = 0; c < CPL; ++c)
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) acc = fmaf((float)kv[u][c][i], qr[c * VEC + i], acc);
-            acc = group_sum<LPR>(acc);
-            s[u] = fmaf(acc, scale, mk[u]); // v = qk*scaler + mask (decoder_kernels.cu:815)
+            s[u] = acc;
+        }
+        group_sum_n<LPR, UNROLL>(s);
+        float tmax = m;
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            s[u] = HAS_MASK ? fmaf(s[u], scale, FAST ? mk[u] * kLog2e : mk[u]) : s[u] * scale;
             if (CHECK && !ok[u]) s[u] = -__builtin_inff();
             tmax = fmaxf(tmax, s[u]);
         }
-        const float alpha = expf(m - tmax);
+        const float alpha = softmax_exp<FAST>(m - tmax);
         m = tmax;
         l *= alpha;
 #pragma unroll
@@ -256,7 +326,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attn_split_kernel(const Par
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             if (CHECK && !ok[u]) continue;
-            const float pr = expf(s[u] - m);
+            const float pr = softmax_exp<FAST>(s[u] - m);
             l += pr;
 #pragma unroll
             for (int c = 0; c < CPL; ++c)
@@ -311,10 +381,11 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attn_split_kernel(const Par
         }
         acc = group_sum<LPR>(acc);
         if (g == 0) {
-            const float s = fmaf(acc, scale, mrow ? mrow[P] : 0.f);
+            const float mk = HAS_MASK ? (FAST ? mrow[P] * kLog2e : mrow[P]) : 0.f;
+            const float s = fmaf(acc, scale, mk);
             const float m_new = fmaxf(m, s);
-            const float alpha = expf(m - m_new);
-            const float pr = expf(s - m_new);
+            const float alpha = softmax_exp<FAST>(m - m_new);
+            const float pr = softmax_exp<FAST>(s - m_new);
             m = m_new;
             l = fmaf(l, alpha, pr);
 #pragma unroll
@@ -338,13 +409,13 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attn_split_kernel(const Par
     __syncthreads();
 
     for (int d = tid; d < D; d += WAVES * 64) {
-        float M = kMaxFloor;
+        float M = floor_m;
 #pragma unroll
         for (int k = 0; k < GROUPS; ++k) M = fmaxf(M, s_m[k]);
         float Lsum = 0.f, O = 0.f;
 #pragma unroll
         for (int k = 0; k < GROUPS; ++k) {
-            const float w = expf(s_m[k] - M);
+            const float w = softmax_exp<FAST>(s_m[k] - M);
             Lsum = fmaf(s_l[k], w, Lsum);
             O = fmaf(s_o[k][d], w, O);
         }
@@ -363,64 +434,146 @@ __global__ __launch_bounds__(WAVES * 64) void decode_attn_split_kernel(const Par
 
 // ---------------------------------------------------------------- combine kernels
 
-// Merged, normalised attention output element d of (b,h) from its split partials.
-__device__ __forceinline__ float merge_partials(const Params &p, int bh, int nsp, int D, int d)
+__device__ __forceinline__ float wave_sum(float x)
 {
-    const size_t slot0 = (size_t)bh * p.split_cap;
-    float M = kMaxFloor;
-    for (int s = 0; s < nsp; ++s) M = fmaxf(M, p.part_m[slot0 + s]);
-    float Lsum = 0.f, O = 0.f;
-    for (int s = 0; s < nsp; ++s) {
-        const float w = expf(p.part_m[slot0 + s] - M);
-        Lsum = fmaf(p.part_l[slot0 + s], w, Lsum);
-        O = fmaf(p.part_o[(slot0 + s) * D + d], w, O);
-    }
-    return O / Lsum;
+    x += dpp_move<0xB1>(x);
+    x += dpp_move<0x4E>(x);
+    x += dpp_move<0x141>(x);
+    x += dpp_move<0x140>(x);
+    x += __shfl_xor(x, 16);
+    x += __shfl_xor(x, 32);
+    return x;
 }
 
-// grid = B*H, block = min(D, 256): out[b, h*D + d] from the partials of (b,h).
-__global__ void decode_attn_combine_kernel(const Params p, int D)
+constexpr int kCombineThreads = 256;
+constexpr int kCombineMaxSplits = 1024;
+
+// grid = B*H, block = 256.  Merges the (m, l, o[D]) partials of one (b,h):
+//   M = max_s m_s;  w_s = exp(m_s - M);  out[d] = sum_s w_s o_s[d] / sum_s w_s l_s.
+// The weights are computed once per split (threads over s), then the weighted sum over splits runs
+// with D/4 threads per split-group (float4 per thread) and 256/(D/4) split-groups side by side, so
+// the partial loads of a group are independent and in flight together.
+template <int D>
+__global__ __launch_bounds__(kCombineThreads) void decode_attn_combine_kernel(const Params p)
 {
-    const int bh = blockIdx.x;
+    constexpr int TPG = D / 4 < kCombineThreads ? D / 4 : kCombineThreads; // threads per split-group
+    constexpr int SG = kCombineThreads / TPG;                             // split-groups
+    constexpr int VPT = D / 4 / TPG;                                      // float4 per thread
+    __shared__ float s_w[kCombineMaxSplits];
+    __shared__ float s_red[2][kCombineThreads / 64];
+    __shared__ float4 s_acc[SG][D / 4];
+
+    const int bh = blockIdx.x, tid = threadIdx.x;
     const int b = bh / p.H;
     const int P = p.pos_per_seq ? p.pos_per_seq[b] : p.start_pos;
-    const bool bad = (P < 0 || P >= p.L);
-    const int nsp = bad ? 0 : (P + p.chunk) / p.chunk; // ceil((P+1)/chunk)
-    for (int d = threadIdx.x; d < D; d += blockDim.x)
-        p.out[(size_t)bh * D + d] = bad ? __builtin_nanf("") : merge_partials(p, bh, nsp, D, d);
+    if (P < 0 || P >= p.L) { // uniform per block
+        for (int d = tid; d < D; d += kCombineThreads) p.out[(size_t)bh * D + d] = __builtin_nanf("");
+        return;
+    }
+    const int nsp = (P + p.chunk) / p.chunk; // ceil((P+1)/chunk) <= split_cap <= kCombineMaxSplits
+    const size_t slot0 = (size_t)bh * p.split_cap;
+    const float floor_m = p.log2_domain ? kMaxFloor * kLog2e : kMaxFloor;
+
+    float mx = floor_m;
+    for (int s = tid; s < nsp; s += kCombineThreads) {
+        const float ms = p.part_m[slot0 + s];
+        s_w[s] = ms;
+        mx = fmaxf(mx, ms);
+    }
+    mx = wave_max(mx);
+    if ((tid & 63) == 0) s_red[0][tid >> 6] = mx;
+    __syncthreads();
+    float M = s_red[0][0];
+#pragma unroll
+    for (int w = 1; w < kCombineThreads / 64; ++w) M = fmaxf(M, s_red[0][w]);
+
+    float lsum = 0.f;
+    for (int s = tid; s < nsp; s += kCombineThreads) {
+        const float dm = s_w[s] - M;
+        const float w = p.log2_domain ? __builtin_amdgcn_exp2f(dm) : expf(dm);
+        s_w[s] = w;
+        lsum = fmaf(p.part_l[slot0 + s], w, lsum);
+    }
+    lsum = wave_sum(lsum);
+    if ((tid & 63) == 0) s_red[1][tid >> 6] = lsum;
+    __syncthreads();
+    float Lsum = s_red[1][0];
+#pragma unroll
+    for (int w = 1; w < kCombineThreads / 64; ++w) Lsum += s_red[1][w];
+
+    const int sg = tid / TPG, t = tid % TPG;
+    float4 acc[VPT];
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) acc[v] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float4 *po = reinterpret_cast<const float4 *>(p.part_o + slot0 * D);
+    int s = sg;
+    for (; s + 3 * SG < nsp; s += 4 * SG) { // four independent partial rows in flight
+        float4 x[4][VPT];
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int v = 0; v < VPT; ++v) x[k][v] = po[(size_t)(s + k * SG) * (D / 4) + v * TPG + t];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float w = s_w[s + k * SG];
+#pragma unroll
+            for (int v = 0; v < VPT; ++v) {
+                acc[v].x = fmaf(x[k][v].x, w, acc[v].x);
+                acc[v].y = fmaf(x[k][v].y, w, acc[v].y);
+                acc[v].z = fmaf(x[k][v].z, w, acc[v].z);
+                acc[v].w = fmaf(x[k][v].w, w, acc[v].w);
+            }
+        }
+    }
+    for (; s < nsp; s += SG) {
+        const float w = s_w[s];
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const float4 x = po[(size_t)s * (D / 4) + v * TPG + t];
+            acc[v].x = fmaf(x.x, w, acc[v].x);
+            acc[v].y = fmaf(x.y, w, acc[v].y);
+            acc[v].z = fmaf(x.z, w, acc[v].z);
+            acc[v].w = fmaf(x.w, w, acc[v].w);
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) s_acc[sg][v * TPG + t] = acc[v];
+    __syncthreads();
+    for (int d4 = tid; d4 < D / 4; d4 += kCombineThreads) {
+        float4 r = s_acc[0][d4];
+#pragma unroll
+        for (int k = 1; k < SG; ++k) {
+            const float4 y = s_acc[k][d4];
+            r.x += y.x; r.y += y.y; r.z += y.z; r.w += y.w;
+        }
+        r.x = r.x / Lsum; r.y = r.y / Lsum; r.z = r.z / Lsum; r.w = r.w / Lsum;
+        reinterpret_cast<float4 *>(p.out + (size_t)bh * D)[d4] = r;
+    }
 }
 
-// grid = B, block = 1024: merge + per-row absmax INT8 quantisation over the H*D outputs of one
-// sequence (launchAttnQuantizedTransposeKernel, decoder_kernels.cu:1179-1212, seq_len == 1):
+// grid = B, block = 1024.  Per-row absmax INT8 quantisation of the attention output of one sequence
+// (launchAttnQuantizedTransposeKernel, decoder_kernels.cu:1179-1212 with seq_len == 1):
 //   absmax = max(-1e9, max |x|); scale[b] = absmax/127; q = sat_s8(rint(x*127/absmax)).
-__global__ __launch_bounds__(1024) void decode_attn_combine_quant_kernel(const Params p, int D)
+// The float output [B, H*D] was written by the streaming or the combine kernel.
+__global__ __launch_bounds__(1024) void attn_quantize_kernel(const float *__restrict__ attn, int8_t *__restrict__ out_q,
+                                                             float *__restrict__ out_scale, int HD)
 {
     __shared__ float s_red[16];
-    const int b = blockIdx.x;
-    const int HD = p.H * D;
-    const int P = p.pos_per_seq ? p.pos_per_seq[b] : p.start_pos;
-    const bool bad = (P < 0 || P >= p.L);
-    const int nsp = bad ? 0 : (P + p.chunk) / p.chunk;
-    const float nan = __builtin_nanf("");
-
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const float *x = attn + (size_t)b * HD;
     float absmax = kMaxFloor;
-    for (int e = threadIdx.x; e < HD; e += blockDim.x) {
-        const float x = bad ? nan : merge_partials(p, b * p.H + e / D, nsp, D, e % D);
-        if (p.out) p.out[(size_t)b * HD + e] = x;
-        absmax = fmaxf(absmax, fabsf(x));
-    }
+    for (int e = tid; e < HD; e += 1024) absmax = fmaxf(absmax, fabsf(x[e]));
     absmax = wave_max(absmax);
-    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = absmax;
+    if ((tid & 63) == 0) s_red[tid >> 6] = absmax;
     __syncthreads();
     absmax = s_red[0];
-    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) absmax = fmaxf(absmax, s_red[w]);
-    if (threadIdx.x == 0) p.out_scale[b] = absmax / 127.0f;
-
-    for (int e = threadIdx.x; e < HD; e += blockDim.x) {
-        const float x = bad ? nan : merge_partials(p, b * p.H + e / D, nsp, D, e % D);
-        const float v = rintf(__fmul_rn(x, 127.0f) / absmax);
-        const int qv = (v != v) ? 0 : (int)fminf(fmaxf(v, -128.f), 127.f);
-        p.out_int8[(size_t)b * HD + e] = (int8_t)qv;
+#pragma unroll
+    for (int w = 1; w < 16; ++w) absmax = fmaxf(absmax, s_red[w]);
+    if (tid == 0) out_scale[b] = absmax / 127.0f;
+    for (int e = tid; e < HD; e += 1024) {
+        const float v = rintf(__fmul_rn(x[e], 127.0f) / absmax);
+        const int qv = (v != v) ? 0 : (int)fminf(fmaxf(v, -128.f), 127.f); // NaN -> 0, saturate
+        out_q[(size_t)b * HD + e] = (int8_t)qv;
     }
 }
 

@@ -16,7 +16,13 @@ using flattn::Params;
 
 thread_local int g_last_hip_error = 0;
 
-constexpr int kWaves = 4;        // 256 threads per streaming workgroup
+#ifndef FLATTN_WAVES
+#define FLATTN_WAVES 4
+#endif
+#ifndef FLATTN_UNROLL
+#define FLATTN_UNROLL 4
+#endif
+constexpr int kWaves = FLATTN_WAVES; // waves per streaming workgroup
 constexpr int kMinChunkRows = 64; // never split a context finer than this
 constexpr int kMaxSplits = 1024;
 
@@ -54,12 +60,12 @@ int validate_desc(const fl_attn_desc *d)
     if (!d) return FL_ATTN_ERR_NULL_POINTER;
     if (d->dtype != FL_ATTN_F32 && d->dtype != FL_ATTN_F16) return FL_ATTN_ERR_DTYPE;
     if (d->batch_size <= 0 || d->head_num <= 0 || d->total_len <= 0) return FL_ATTN_ERR_SHAPE;
-    if (d->batch_size > 65535 || d->head_num > 65535) return FL_ATTN_ERR_SHAPE; // grid y/z limits
+    if (d->batch_size > 65535 || d->head_num > 65535) return FL_ATTN_ERR_SHAPE;
     if (!head_dim_ok(d->size_per_head)) return FL_ATTN_ERR_HEAD_DIM;
     if (d->nsplit < 0 || d->nsplit > kMaxSplits || d->reserved != 0) return FL_ATTN_ERR_ARGUMENT;
     if (!(d->softmax_scale >= 0.f) || std::isinf(d->softmax_scale)) return FL_ATTN_ERR_ARGUMENT;
-    // element counts of a cache must stay addressable with a 64-bit byte offset; B*H must fit int
-    if ((int64_t)d->batch_size * d->head_num > (int64_t)INT32_MAX / 2) return FL_ATTN_ERR_SHAPE;
+    // the streaming grid is one-dimensional: B*H*splits workgroups must fit the 2^31 limit
+    if ((int64_t)d->batch_size * d->head_num > (int64_t)INT32_MAX / kMaxSplits) return FL_ATTN_ERR_SHAPE;
     return FL_ATTN_OK;
 }
 
@@ -77,42 +83,77 @@ int unroll_for(const fl_attn_desc *d)
     const int vec = d->dtype == FL_ATTN_F16 ? 8 : 4;
     const int ch = d->size_per_head / vec;
     const int cpl = ch <= 64 ? 1 : ch / 64;
-    return cpl >= 4 ? 1 : (cpl == 2 ? 2 : 4);
+    return cpl >= 4 ? 1 : (cpl == 2 ? 2 : FLATTN_UNROLL);
 }
 
-// Upper bound of splits for any context of this shape: sizes the workspace.
-int split_cap(const fl_attn_desc *d)
+// ---- launch planning ---------------------------------------------------------------------------
+// slots = workgroups the device holds at once (8 four-wave workgroups per CU at 64 VGPRs).
+// Uniform batches: when B*H fills the slots, one split per (b,h) (no partials, no combine pass) unless
+// a fractional last round of workgroups would idle much of the chip, in which case 2-4 splits smooth
+// it; when B*H is smaller, floor(slots / (B*H)) splits fill the device in a single round.
+// Ragged batches (per-sequence positions on the device): work per (b,h) varies, so splits are also
+// capped at ~256 KB of K+V per workgroup, which measured best on 13B-shaped ragged batches.
+constexpr size_t kRaggedChunkBytes = 256 * 1024;
+
+int row_bytes(const fl_attn_desc *d) { return d->size_per_head * (d->dtype == FL_ATTN_F16 ? 2 : 4); }
+
+int min_chunk_rows(const fl_attn_desc *d)
 {
-    if (d->nsplit > 0) return d->nsplit;
+    const int tile = rows_per_tile(d, unroll_for(d));
+    return tile > kMinChunkRows ? tile : kMinChunkRows;
+}
+
+int uniform_splits(const fl_attn_desc *d, int ctx)
+{
     const int64_t bh = (int64_t)d->batch_size * d->head_num;
-    const int64_t target = (int64_t)device_cus() * 8;
-    int64_t want = (target + bh - 1) / bh;
-    int64_t most = ((int64_t)d->total_len + kMinChunkRows - 1) / kMinChunkRows;
-    int64_t n = want < most ? want : most;
+    const int64_t slots = (int64_t)device_cus() * 8;
+    int64_t n;
+    if (bh <= slots) {
+        n = slots / bh;
+    } else {
+        // estimated cost of n splits: idle fraction of the last round, plus ~2% for the combine pass
+        double best = 1e30;
+        n = 1;
+        for (int c = 1; c <= 4; ++c) {
+            const double rounds = (double)(bh * c) / (double)slots;
+            const double cost = std::ceil(rounds) / rounds * (c > 1 ? 1.02 : 1.0);
+            if (cost < best - 1e-9) { best = cost; n = c; }
+        }
+    }
+    const int64_t most = ((int64_t)ctx + min_chunk_rows(d) - 1) / min_chunk_rows(d);
+    if (n > most) n = most;
     if (n < 1) n = 1;
     if (n > kMaxSplits) n = kMaxSplits;
     return (int)n;
 }
 
-void make_plan(const fl_attn_desc *d, int ctx, fl_attn_plan *plan)
+int ragged_splits(const fl_attn_desc *d, int max_ctx)
+{
+    const int64_t by_bytes = ((int64_t)max_ctx * 2 * row_bytes(d) + kRaggedChunkBytes - 1) / (int64_t)kRaggedChunkBytes;
+    int64_t n = uniform_splits(d, max_ctx);
+    if (by_bytes > n) n = by_bytes;
+    const int64_t most = ((int64_t)max_ctx + min_chunk_rows(d) - 1) / min_chunk_rows(d);
+    if (n > most) n = most;
+    if (n < 1) n = 1;
+    if (n > kMaxSplits) n = kMaxSplits;
+    return (int)n;
+}
+
+// Upper bound of splits for any call with this shape (both estimates grow with the context length
+// and the ragged one dominates): sizes the workspace.
+int split_cap(const fl_attn_desc *d)
+{
+    if (d->nsplit > 0) return d->nsplit;
+    return ragged_splits(d, d->total_len);
+}
+
+void make_plan(const fl_attn_desc *d, int ctx, bool ragged, fl_attn_plan *plan)
 {
     const int tile = rows_per_tile(d, unroll_for(d));
-    int n;
-    if (d->nsplit > 0) {
-        n = d->nsplit;
-    } else {
-        const int64_t bh = (int64_t)d->batch_size * d->head_num;
-        const int64_t target = (int64_t)device_cus() * 8;
-        int64_t want = (target + bh - 1) / bh;
-        int64_t most = ((int64_t)ctx + kMinChunkRows - 1) / kMinChunkRows;
-        int64_t nn = want < most ? want : most;
-        if (nn < 1) nn = 1;
-        if (nn > kMaxSplits) nn = kMaxSplits;
-        n = (int)nn;
-    }
+    int n = d->nsplit > 0 ? d->nsplit : (ragged ? ragged_splits(d, ctx) : uniform_splits(d, ctx));
     if (n > ctx) n = ctx > 0 ? ctx : 1;
     int chunk = (ctx + n - 1) / n;
-    if (d->nsplit == 0) chunk = (chunk + tile - 1) / tile * tile; // whole tiles per split
+    if (chunk > tile) chunk = (chunk + tile - 1) / tile * tile; // whole tiles per split (may lower nsplit)
     if (chunk < 1) chunk = 1;
     plan->chunk_rows = chunk;
     plan->nsplit = (ctx + chunk - 1) / chunk;
@@ -122,13 +163,49 @@ void make_plan(const fl_attn_desc *d, int ctx, fl_attn_plan *plan)
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
-size_t workspace_need(const fl_attn_desc *d)
+// Workspace layout: [float output B*H*D (used when the caller asks for INT8 only)]
+//                   [part_o slots*D] [part_m slots] [part_l slots], each 256-byte aligned.
+struct WorkspaceLayout {
+    size_t tmp_out, part_o, part_m, part_l, total;
+};
+
+WorkspaceLayout workspace_layout(const fl_attn_desc *d)
 {
     const size_t slots = (size_t)d->batch_size * d->head_num * (size_t)split_cap(d);
-    const size_t part_o = align_up(slots * d->size_per_head * sizeof(float), 256);
-    const size_t part_ml = align_up(slots * sizeof(float), 256);
-    return part_o + 2 * part_ml;
+    WorkspaceLayout w;
+    w.tmp_out = 0;
+    w.part_o = align_up((size_t)d->batch_size * d->head_num * d->size_per_head * sizeof(float), 256);
+    w.part_m = w.part_o + align_up(slots * d->size_per_head * sizeof(float), 256);
+    w.part_l = w.part_m + align_up(slots * sizeof(float), 256);
+    w.total = w.part_l + align_up(slots * sizeof(float), 256);
+    return w;
 }
+
+size_t workspace_need(const fl_attn_desc *d) { return workspace_layout(d).total; }
+
+template <int D>
+void launch_combine(const Params &p, int bh, hipStream_t stream)
+{
+    hipLaunchKernelGGL((flattn::decode_attn_combine_kernel<D>), dim3(bh), dim3(flattn::kCombineThreads), 0, stream, p);
+}
+
+hipError_t dispatch_combine(int D, const Params &p, int bh, hipStream_t stream)
+{
+    switch (D) {
+    case 32: launch_combine<32>(p, bh, stream); break;
+    case 64: launch_combine<64>(p, bh, stream); break;
+    case 128: launch_combine<128>(p, bh, stream); break;
+    case 256: launch_combine<256>(p, bh, stream); break;
+    case 512: launch_combine<512>(p, bh, stream); break;
+    case 1024: launch_combine<1024>(p, bh, stream); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// fp16 storage streams half the bytes per row, so its softmax uses the one-instruction base-2
+// exponential; fp32 storage (the reference's cache type) keeps expf.
+template <typename T> constexpr bool kFastExp = std::is_same<T, _Float16>::value;
 
 template <typename T, int D>
 hipError_t launch_split(const Params &p, dim3 grid, hipStream_t stream)
@@ -136,9 +213,13 @@ hipError_t launch_split(const Params &p, dim3 grid, hipStream_t stream)
     constexpr int VEC = flattn::Vec16<T>::N;
     constexpr int CH = D / VEC;
     constexpr int CPL = CH <= 64 ? 1 : CH / 64;
-    constexpr int UNROLL = CPL >= 4 ? 1 : (CPL == 2 ? 2 : 4);
-    hipLaunchKernelGGL((flattn::decode_attn_split_kernel<T, D, kWaves, UNROLL>), grid, dim3(kWaves * 64), 0,
-                       stream, p);
+    constexpr int UNROLL = CPL >= 4 ? 1 : (CPL == 2 ? 2 : FLATTN_UNROLL);
+    if (p.attn_mask)
+        hipLaunchKernelGGL((flattn::decode_attn_split_kernel<T, D, kWaves, UNROLL, true, kFastExp<T>>), grid,
+                           dim3(kWaves * 64), 0, stream, p);
+    else
+        hipLaunchKernelGGL((flattn::decode_attn_split_kernel<T, D, kWaves, UNROLL, false, kFastExp<T>>), grid,
+                           dim3(kWaves * 64), 0, stream, p);
     return hipGetLastError();
 }
 
@@ -202,13 +283,13 @@ int fl_kv_cache_bytes(const fl_attn_desc *desc, size_t *bytes)
     return FL_ATTN_OK;
 }
 
-int fl_decode_attn_plan(const fl_attn_desc *desc, int32_t ctx, fl_attn_plan *plan)
+int fl_decode_attn_plan(const fl_attn_desc *desc, int32_t ctx, int32_t ragged, fl_attn_plan *plan)
 {
     if (!plan) return FL_ATTN_ERR_NULL_POINTER;
     int st = validate_desc(desc);
     if (st != FL_ATTN_OK) return st;
     if (ctx < 1 || ctx > desc->total_len) return FL_ATTN_ERR_POSITION;
-    make_plan(desc, ctx, plan);
+    make_plan(desc, ctx, ragged != 0, plan);
     return FL_ATTN_OK;
 }
 
@@ -247,57 +328,54 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
     if (io->attn_mask && io->mask_ld < 0) return FL_ATTN_ERR_ARGUMENT;
 
     fl_attn_plan plan;
-    make_plan(desc, max_pos + 1, &plan);
+    make_plan(desc, max_pos + 1, ragged, &plan);
     const int cap = split_cap(desc);
     if (plan.nsplit > cap) return FL_ATTN_ERR_ARGUMENT;
 
-    const bool direct = plan.nsplit == 1 && !quant;
-    const size_t need = workspace_need(desc);
-    if (!direct) {
-        if (!io->workspace || io->workspace_bytes < need) return FL_ATTN_ERR_WORKSPACE;
+    const bool direct = plan.nsplit == 1; // the streaming kernel normalises and writes the output itself
+    const bool need_ws = !direct || (quant && !io->out);
+    const WorkspaceLayout wl = workspace_layout(desc);
+    if (need_ws) {
+        if (!io->workspace || io->workspace_bytes < wl.total) return FL_ATTN_ERR_WORKSPACE;
         if ((reinterpret_cast<uintptr_t>(io->workspace) & 255u) != 0) return FL_ATTN_ERR_WORKSPACE;
     }
 
     const int D = desc->size_per_head;
+    char *ws = static_cast<char *>(io->workspace);
     Params p{};
     p.q = io->q; p.k_new = io->k_new; p.v_new = io->v_new;
     p.k_cache = io->k_cache; p.v_cache = io->v_cache;
     p.freq_cis = io->freq_cis; p.attn_mask = io->attn_mask; p.pos_per_seq = io->start_pos_per_seq;
-    p.out = io->out;
+    p.out = io->out ? io->out : reinterpret_cast<float *>(ws + wl.tmp_out);
     if (!direct) {
-        const size_t slots = (size_t)desc->batch_size * desc->head_num * (size_t)cap;
-        const size_t part_o = align_up(slots * D * sizeof(float), 256);
-        const size_t part_ml = align_up(slots * sizeof(float), 256);
-        char *ws = static_cast<char *>(io->workspace);
-        p.part_o = reinterpret_cast<float *>(ws);
-        p.part_m = reinterpret_cast<float *>(ws + part_o);
-        p.part_l = reinterpret_cast<float *>(ws + part_o + part_ml);
+        p.part_o = reinterpret_cast<float *>(ws + wl.part_o);
+        p.part_m = reinterpret_cast<float *>(ws + wl.part_m);
+        p.part_l = reinterpret_cast<float *>(ws + wl.part_l);
     }
     p.inp_scale = io->qkv_inp_scale; p.wq_scale = io->q_weight_scale;
     p.wk_scale = io->k_weight_scale; p.wv_scale = io->v_weight_scale;
-    p.out_int8 = io->out_int8; p.out_scale = io->out_scale;
     p.mask_ld = io->mask_ld;
     p.B = desc->batch_size; p.H = desc->head_num; p.L = L;
     p.start_pos = io->start_pos; p.rope_row = io->rope_row;
     p.chunk = plan.chunk_rows; p.split_cap = cap; p.direct = direct ? 1 : 0;
     p.scale = desc->softmax_scale > 0.f ? desc->softmax_scale : 1.0f / sqrtf((float)D);
+    p.log2_domain = desc->dtype == FL_ATTN_F16 ? 1 : 0;
 
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    const int bh = desc->batch_size * desc->head_num;
     if (passes & 1) {
-        dim3 grid(plan.nsplit, desc->head_num, desc->batch_size);
+        dim3 grid((unsigned)plan.nsplit * (unsigned)bh);
         hipError_t e = desc->dtype == FL_ATTN_F16 ? dispatch_split<_Float16>(D, p, grid, stream)
                                                   : dispatch_split<float>(D, p, grid, stream);
         if (!check_hip(e)) return FL_ATTN_ERR_HIP;
     }
-    if ((passes & 2) && !direct) {
+    if (passes & 2) {
+        if (!direct && !check_hip(dispatch_combine(D, p, bh, stream))) return FL_ATTN_ERR_HIP;
         if (quant) {
-            hipLaunchKernelGGL(flattn::decode_attn_combine_quant_kernel, dim3(desc->batch_size), dim3(1024), 0,
-                               stream, p, D);
-        } else {
-            hipLaunchKernelGGL(flattn::decode_attn_combine_kernel, dim3(desc->batch_size * desc->head_num),
-                               dim3(D < 256 ? D : 256), 0, stream, p, D);
+            hipLaunchKernelGGL(flattn::attn_quantize_kernel, dim3(desc->batch_size), dim3(1024), 0, stream, p.out,
+                               io->out_int8, io->out_scale, desc->head_num * D);
+            if (!check_hip(hipGetLastError())) return FL_ATTN_ERR_HIP;
         }
-        if (!check_hip(hipGetLastError())) return FL_ATTN_ERR_HIP;
     }
     return FL_ATTN_OK;
 }

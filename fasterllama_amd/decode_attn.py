@@ -42,10 +42,10 @@ class DecodeAttention:
         # torch allocations are 512-byte aligned; the library asks for 256
         self.workspace = torch.empty(max(n.value, 256), dtype=torch.uint8, device=self.device)
 
-    def plan(self, ctx: int) -> capi.AttnPlan:
+    def plan(self, ctx: int, ragged: bool = False) -> capi.AttnPlan:
         plan = capi.AttnPlan()
         with torch.cuda.device(self.device):
-            capi.check(self.lib.fl_decode_attn_plan(C.byref(self.desc), ctx, C.byref(plan)))
+            capi.check(self.lib.fl_decode_attn_plan(C.byref(self.desc), ctx, int(ragged), C.byref(plan)))
         return plan
 
     def make_io(self, q, k_new, v_new, k_cache, v_cache, freq_cis, out, start_pos: int = 0,

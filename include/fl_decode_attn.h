@@ -116,8 +116,9 @@ typedef struct fl_attn_plan {
  * (open_decoder.cu:54-67: query_out_buf_, key_out_buf_, value_out_fp_buf_, qk_buf_). */
 int fl_decode_attn_workspace_bytes(const fl_attn_desc *desc, size_t *bytes);
 
-/* The plan for a given context length (for logging and for the benchmark's byte accounting). */
-int fl_decode_attn_plan(const fl_attn_desc *desc, int32_t ctx, fl_attn_plan *plan);
+/* The plan for a given context length (for logging and for the benchmark's byte accounting).
+ * ragged != 0: the plan used when start_pos_per_seq is given and ctx = max_start_pos + 1. */
+int fl_decode_attn_plan(const fl_attn_desc *desc, int32_t ctx, int32_t ragged, fl_attn_plan *plan);
 
 /* One decode step of attention for all (batch, head) pairs. */
 int fl_decode_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream);

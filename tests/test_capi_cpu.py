@@ -80,7 +80,7 @@ def test_null_arguments():
     assert lib.fl_decode_attn_workspace_bytes(None, C.byref(n)) == capi.FL_ATTN_ERR_NULL_POINTER
     assert lib.fl_decode_attn_workspace_bytes(C.byref(desc()), None) == capi.FL_ATTN_ERR_NULL_POINTER
     assert lib.fl_decode_attn_forward(C.byref(desc()), None, None) == capi.FL_ATTN_ERR_NULL_POINTER
-    assert lib.fl_decode_attn_plan(C.byref(desc()), 8, None) == capi.FL_ATTN_ERR_NULL_POINTER
+    assert lib.fl_decode_attn_plan(C.byref(desc()), 8, 0, None) == capi.FL_ATTN_ERR_NULL_POINTER
     assert lib.fl_rope_table(None, 8, 64, 10000.0, None) == capi.FL_ATTN_ERR_NULL_POINTER
     for name in ("q", "k_new", "v_new", "k_cache", "v_cache", "freq_cis", "out"):
         assert lib.fl_decode_attn_forward(C.byref(desc()), C.byref(fake_io(**{name: None})), None) \
@@ -131,20 +131,40 @@ def test_plans_cover_the_context_and_respect_forced_splits():
         for ctx in (1, 2, 63, 64, 65, 1000, L):
             if ctx > L:
                 continue
-            assert lib.fl_decode_attn_plan(C.byref(d), ctx, C.byref(plan)) == 0
-            assert plan.nsplit >= 1 and plan.chunk_rows >= 1
-            assert plan.nsplit * plan.chunk_rows >= ctx > (plan.nsplit - 1) * plan.chunk_rows
-            assert plan.two_pass == (1 if plan.nsplit > 1 else 0)
-            cap = max(cap or 0, plan.nsplit)
+            for ragged in (0, 1):
+                assert lib.fl_decode_attn_plan(C.byref(d), ctx, ragged, C.byref(plan)) == 0
+                assert plan.nsplit >= 1 and plan.chunk_rows >= 1
+                assert plan.nsplit * plan.chunk_rows >= ctx > (plan.nsplit - 1) * plan.chunk_rows
+                assert plan.two_pass == (1 if plan.nsplit > 1 else 0)
+                cap = max(cap or 0, plan.nsplit)
         # the workspace sized from the shape alone covers the largest plan
         n = C.c_size_t(0)
         assert lib.fl_decode_attn_workspace_bytes(C.byref(d), C.byref(n)) == 0
         assert n.value >= B * H * cap * (d.size_per_head + 2) * 4
     d = desc(B=1, H=2, L=4096, nsplit=7)
-    assert lib.fl_decode_attn_plan(C.byref(d), 4096, C.byref(plan)) == 0 and plan.nsplit == 7
-    assert lib.fl_decode_attn_plan(C.byref(d), 3, C.byref(plan)) == 0 and plan.nsplit == 3  # never more splits than rows
-    assert lib.fl_decode_attn_plan(C.byref(d), 0, C.byref(plan)) == capi.FL_ATTN_ERR_POSITION
-    assert lib.fl_decode_attn_plan(C.byref(d), 4097, C.byref(plan)) == capi.FL_ATTN_ERR_POSITION
+    assert lib.fl_decode_attn_plan(C.byref(d), 4096, 0, C.byref(plan)) == 0 and plan.nsplit == 7
+    assert lib.fl_decode_attn_plan(C.byref(d), 3, 0, C.byref(plan)) == 0 and plan.nsplit == 3  # never more splits than rows
+    assert lib.fl_decode_attn_plan(C.byref(d), 0, 0, C.byref(plan)) == capi.FL_ATTN_ERR_POSITION
+    assert lib.fl_decode_attn_plan(C.byref(d), 4097, 0, C.byref(plan)) == capi.FL_ATTN_ERR_POSITION
+
+
+def test_plan_heuristics_at_the_benchmark_shapes():
+    """Without a GPU the library assumes 256 compute units (2048 resident workgroups)."""
+    lib = capi.load()
+    plan = capi.AttnPlan()
+    # headline: B*H = 2048 fills the device -> single pass, no partials
+    d = desc(B=64, H=32, D=128, L=2048)
+    assert lib.fl_decode_attn_plan(C.byref(d), 2048, 0, C.byref(plan)) == 0 and (plan.nsplit, plan.two_pass) == (1, 0)
+    # B=8: 256 (b,h) pairs -> 8 splits of 128 rows fill the device in one round
+    d = desc(B=8, H=32, D=128, L=1024)
+    assert lib.fl_decode_attn_plan(C.byref(d), 1024, 0, C.byref(plan)) == 0 and (plan.nsplit, plan.chunk_rows) == (8, 128)
+    # B=1, ctx 4096: 64 splits of 64 rows
+    d = desc(B=1, H=32, D=128, L=4096)
+    assert lib.fl_decode_attn_plan(C.byref(d), 4096, 0, C.byref(plan)) == 0 and (plan.nsplit, plan.chunk_rows) == (64, 64)
+    # ragged 13B batch: ~256 KB of K+V per workgroup -> 512-row chunks
+    d = desc(B=32, H=40, D=128, L=4096)
+    assert lib.fl_decode_attn_plan(C.byref(d), 4096, 1, C.byref(plan)) == 0 and (plan.nsplit, plan.chunk_rows) == (8, 512)
+    assert lib.fl_decode_attn_plan(C.byref(d), 4096, 0, C.byref(plan)) == 0 and plan.nsplit == 1
 
 
 def test_kv_cache_bytes_uses_64_bit_sizes():
