@@ -40,7 +40,10 @@ HEADLINE = "cfg3"
 # HBM bytes per launch of the streaming kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
 # scaled by the factor the same counters read for a copy kernel of known size.  Filled in from
 # the summaries under profiles/ (None until measured for that workload).
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/decode_attn_split_kernel_f16_b64_h32_d128_ctx2048.md
+    "cfg3": 2150680000,
+}
 
 
 def algorithmic_bytes(B, H, D, e, sum_ctx, has_mask=False, mean_ctx=0):
