@@ -31,7 +31,7 @@ WORKLOADS = {
     "cfg3": dict(B=64, H=32, D=128, ctx=2048, L=2048, dtype="f16", copies=1),
     "cfg4": dict(B=1, H=32, D=128, ctx=4096, L=4096, dtype="f16", copies=12),
     "cfg5": dict(B=32, H=40, D=128, ctx=None, L=4096, dtype="f16", copies=1, ragged=True),
-    # exploration shapes (not BASELINE configurations)
+    # exploration shapes (not among the five headline configurations)
     "x13b_uniform": dict(B=32, H=40, D=128, ctx=4096, L=4096, dtype="f16", copies=1),
     "x7b_halffull": dict(B=64, H=32, D=128, ctx=2048, L=4096, dtype="f16", copies=1),
 }

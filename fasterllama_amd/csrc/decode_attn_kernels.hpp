@@ -233,48 +233,23 @@ void decode_attn_split_kernel(const Params p)
     const int g = lane / LPR, lig = lane % LPR;
     const int group = wave * GPW + g;
 
-    const bool is_i32 = p.inp_scale != nullptr;
-    const float inp_scale = is_i32 ? p.inp_scale[b] : 0.f;
-    const int rope_row = p.rope_row < 0 ? P : p.rope_row;
-    const float *freq = p.freq_cis + (size_t)rope_row * D;
-
-    // RoPE(q) for the dims this lane owns, kept in registers (fp32)
-    float qr[EPL];
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) {
-        const int e0 = (c * LPR + lig) * VEC;
-        float x[VEC];
-        load_token_chunk<T, VEC>(p.q, (size_t)bh * D + e0, is_i32, inp_scale,
-                                 is_i32 ? p.wq_scale + h * D + e0 : nullptr, x);
-#pragma unroll
-        for (int i = 0; i < VEC; i += 4) {
-            float4 f = *reinterpret_cast<const float4 *>(freq + e0 + i);
-            rope_pair(x[i], x[i + 1], f.x, f.y, qr[c * VEC + i], qr[c * VEC + i + 1]);
-            rope_pair(x[i + 2], x[i + 3], f.z, f.w, qr[c * VEC + i + 2], qr[c * VEC + i + 3]);
-        }
-    }
-
     // Uniform (scalar) base of this (b,h) plus a 32-bit per-lane byte offset: the loads below are
     // "scalar base + vector offset" with no per-row 64-bit vector address arithmetic.
     const char *Kb = reinterpret_cast<const char *>(p.k_cache) + (size_t)bh * L * ROW_BYTES;
     const char *Vb = reinterpret_cast<const char *>(p.v_cache) + (size_t)bh * L * ROW_BYTES;
     const uint32_t lane_off = (uint32_t)(group * ROW_BYTES + lig * 16);
     const float *mrow = HAS_MASK ? p.attn_mask + (size_t)P * p.mask_ld : nullptr;
-    // v = qk*scaler + mask (decoder_kernels.cu:815); the base-2 path folds log2(e) into both terms
-    const float scale = FAST ? p.scale * kLog2e : p.scale;
-    const float floor_m = FAST ? kMaxFloor * kLog2e : kMaxFloor;
-
-    float m = floor_m, l = 0.f;
-    float o[EPL];
-#pragma unroll
-    for (int e = 0; e < EPL; ++e) o[e] = 0.f;
 
     // One tile = UNROLL rows per lane-group.  CHECK guards the ragged last tile.
-    auto tile = [&](int r0, auto check_tag) {
+    V kv[UNROLL][CPL], vv[UNROLL][CPL];
+    float mk[UNROLL];
+    bool ok[UNROLL];
+    constexpr int ROWS_PER_TILE = GROUPS * UNROLL;
+
+    // Issues every load of the tile that starts at row r0 and fences the scheduler so that all
+    // 2*UNROLL*CPL of them stay in flight together.
+    auto issue_tile = [&](int r0, auto check_tag) {
         constexpr bool CHECK = decltype(check_tag)::value;
-        V kv[UNROLL][CPL], vv[UNROLL][CPL];
-        float mk[UNROLL];
-        bool ok[UNROLL];
         const char *kt = Kb + (size_t)r0 * ROW_BYTES; // uniform
         const char *vt = Vb + (size_t)r0 * ROW_BYTES;
 #pragma unroll
@@ -300,6 +275,42 @@ void decode_attn_split_kernel(const Params p)
             for (int c = 0; c < CPL; ++c)
                 vv[u][c] = __builtin_nontemporal_load(reinterpret_cast<const V *>(vt + off + c * LPR * 16));
         }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    const bool is_i32 = p.inp_scale != nullptr;
+    const float inp_scale = is_i32 ? p.inp_scale[b] : 0.f;
+    const int rope_row = p.rope_row < 0 ? P : p.rope_row;
+    const float *freq = p.freq_cis + (size_t)rope_row * D;
+
+    // RoPE(q) for the dims this lane owns, kept in registers (fp32)
+    float qr[EPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+        const int e0 = (c * LPR + lig) * VEC;
+        float x[VEC];
+        load_token_chunk<T, VEC>(p.q, (size_t)bh * D + e0, is_i32, inp_scale,
+                                 is_i32 ? p.wq_scale + h * D + e0 : nullptr, x);
+#pragma unroll
+        for (int i = 0; i < VEC; i += 4) {
+            float4 f = *reinterpret_cast<const float4 *>(freq + e0 + i);
+            rope_pair(x[i], x[i + 1], f.x, f.y, qr[c * VEC + i], qr[c * VEC + i + 1]);
+            rope_pair(x[i + 2], x[i + 3], f.z, f.w, qr[c * VEC + i + 2], qr[c * VEC + i + 3]);
+        }
+    }
+
+    // v = qk*scaler + mask (decoder_kernels.cu:815); the base-2 path folds log2(e) into both terms
+    const float scale = FAST ? p.scale * kLog2e : p.scale;
+    const float floor_m = FAST ? kMaxFloor * kLog2e : kMaxFloor;
+
+    float m = floor_m, l = 0.f;
+    float o[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) o[e] = 0.f;
+
+    // Scores, online-softmax update and weighted V sum for the tile held in kv/vv.
+    auto consume_tile = [&](auto check_tag) {
+        constexpr bool CHECK = decltype(check_tag)::value;
         float s[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
@@ -336,10 +347,18 @@ void decode_attn_split_kernel(const Params p)
         }
     };
 
-    constexpr int ROWS_PER_TILE = GROUPS * UNROLL;
+    // (Issuing the first tile before q is fetched and rotated was tried: it saves one memory latency
+    // per workgroup but keeps 32 more registers live across the prologue, and the spills it causes at
+    // 64 VGPRs cost more than the latency saved: 310 -> 331 us at B=64, H=32, ctx=2048.)
     int r = start;
-    for (; r + ROWS_PER_TILE <= cache_end; r += ROWS_PER_TILE) tile(r, std::false_type{});
-    if (r < cache_end) tile(r, std::true_type{});
+    for (; r + ROWS_PER_TILE <= cache_end; r += ROWS_PER_TILE) {
+        issue_tile(r, std::false_type{});
+        consume_tile(std::false_type{});
+    }
+    if (r < cache_end) {
+        issue_tile(r, std::true_type{});
+        consume_tile(std::true_type{});
+    }
 
     // The new token: RoPE(k_new) and v_new are rounded to the storage type, appended at row P
     // (decoder_kernels.cu:605-610) and attended to from registers.  Every group of wave 0
