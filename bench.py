@@ -61,7 +61,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS) + ["all"],
+                    help="'all' prints one JSON line per configuration cfg1..cfg5 (each in a child process)")
     ap.add_argument("--nsplit", type=int, default=0, help="force the context split count (0 = library's choice)")
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -70,6 +71,15 @@ def main() -> int:
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings), then exit")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
     args = ap.parse_args()
+
+    if args.workload == "all":
+        import subprocess
+        rc = 0
+        for w in ("cfg1", "cfg2", "cfg3", "cfg4", "cfg5"):
+            cmd = [sys.executable, os.path.abspath(__file__), "--workload", w, "--steps", str(args.steps),
+                   "--warmup", str(args.warmup), "--seed", str(args.seed)] + (["--no-cpu"] if args.no_cpu else [])
+            rc |= subprocess.run(cmd).returncode
+        return rc
 
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no cross-GPU exchange); "

@@ -122,6 +122,9 @@ int uniform_splits(const fl_attn_desc *d, int ctx)
     }
     const int64_t most = ((int64_t)ctx + min_chunk_rows(d) - 1) / min_chunk_rows(d);
     if (n > most) n = most;
+    // a combine launch costs about as much as streaming three more tiles in one workgroup
+    // (measured 5.1 us unsplit vs 7.7 us split at B=1, H=4, ctx=128): short contexts stay whole
+    if (ctx <= 4 * min_chunk_rows(d)) n = 1;
     if (n < 1) n = 1;
     if (n > kMaxSplits) n = kMaxSplits;
     return (int)n;

@@ -243,3 +243,66 @@ def test_forward_reports_errors_instead_of_exiting(gpu):
     out = op.forward(q, q, q, kc, kc, f, start_pos=3)  # still usable afterwards
     torch.cuda.synchronize()
     assert torch.isfinite(out).all()
+
+
+# ----------------------------------------------------------------------------- extreme plans and offsets
+
+@pytest.mark.parametrize("ctx,nsplit", [(100, 64), (4096, 1024), (777, 13), (65, 65)])
+def test_forced_tiny_chunks(gpu, ctx, nsplit):
+    # chunks of 1-6 rows: every workgroup runs only the bounds-checked tile
+    c = Case(1, 4, 128, 4096, "f16", start_pos=ctx - 1, seed=ctx)
+    check(c, gpu, nsplit=nsplit, what=f"ctx={ctx} nsplit={nsplit}")
+
+
+def test_mask_with_custom_row_stride_and_ragged_positions(gpu):
+    import torch
+    from fasterllama_amd.decode_attn import DecodeAttention
+    B, H, D, L, ld = 4, 3, 128, 96, 128  # mask rows padded to 128 floats
+    lens = np.array([96, 5, 40, 77])
+    mask = (np.random.default_rng(5).standard_normal((L, ld)) * 3).astype(np.float32)
+    c = Case(B, H, D, L, "f16", lens=lens, pad=np.nan)
+    kc, vc = c.k_cache.copy(), c.v_cache.copy()
+    want = ref.decode_attn(c.q, c.k_new, c.v_new, kc, vc, c.freq, attn_mask=mask, mask_ld=ld,
+                           start_pos_per_seq=lens - 1, acc_double=True)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+    op = DecodeAttention(B, H, D, L, torch.float16, device=gpu)
+    kc_d, vc_d = t(c.k_cache), t(c.v_cache)
+    out = op.forward(t(c.q), t(c.k_new), t(c.v_new), kc_d, vc_d, t(c.freq), attn_mask=t(mask), mask_ld=ld,
+                     start_pos_per_seq=t((lens - 1).astype(np.int32)), max_start_pos=95)
+    torch.cuda.synchronize()
+    assert_cache_bit_exact(kc_d.cpu().numpy(), kc, "k_cache")
+    assert_out_close(out.cpu().numpy(), want, "f16", "mask_ld=128 ragged")
+
+
+def test_byte_offsets_beyond_4_gib(gpu):
+    """fp32 caches of 4 GiB each (B=64, H=32, L=4096, D=128): byte offsets of the last sequences
+    exceed 2^32 and element offsets 2^30.  The oracle checks the first and the last sequence."""
+    import torch
+    from fasterllama_amd.decode_attn import DecodeAttention
+    B, H, D, L, P = 64, 32, 128, 4096, 1500
+    q = synth.normal((B, 1, H, D), np.float32, synth.TENSOR_Q)
+    k = synth.normal((B, 1, H, D), np.float32, synth.TENSOR_K_NEW)
+    v = synth.normal((B, 1, H, D), np.float32, synth.TENSOR_V_NEW)
+    freq = synth.freq_cis_table(L, D)
+    kc_d = torch.empty(B, H, L, D, dtype=torch.float32, device=gpu)
+    vc_d = torch.empty_like(kc_d)
+    host = {}
+    per_seq = H * L * D
+    for b in range(B):  # fill sequence by sequence: only two sequences are kept on the host
+        kb = synth.normal((1, H, L, D), np.float32, synth.TENSOR_K_CACHE, index0=b * per_seq)
+        vb = synth.normal((1, H, L, D), np.float32, synth.TENSOR_V_CACHE, index0=b * per_seq)
+        kc_d[b:b + 1].copy_(torch.from_numpy(kb))
+        vc_d[b:b + 1].copy_(torch.from_numpy(vb))
+        if b in (0, B - 1):
+            host[b] = (kb, vb)
+    op = DecodeAttention(B, H, D, L, torch.float32, device=gpu)
+    t = lambda a: torch.from_numpy(a).to(gpu)
+    out = op.forward(t(q), t(k), t(v), kc_d, vc_d, t(freq), start_pos=P)
+    torch.cuda.synchronize()
+    out_h = out.cpu().numpy()
+    assert np.isfinite(out_h).all()
+    for b, (kb, vb) in host.items():
+        want = ref.decode_attn(q[b:b + 1], k[b:b + 1], v[b:b + 1], kb, vb, freq, start_pos=P, acc_double=True, threads=16)
+        assert_out_close(out_h[b:b + 1], want, "f32", f"sequence {b}")
+        assert_cache_bit_exact(kc_d[b:b + 1].cpu().numpy(), kb, f"k_cache of sequence {b}")
+        assert_cache_bit_exact(vc_d[b:b + 1].cpu().numpy(), vb, f"v_cache of sequence {b}")
