@@ -70,6 +70,10 @@ def main() -> int:
                     help="only run a plain 1 GiB -> 1 GiB elementwise copy kernel a few times (for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings), then exit")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
+    ap.add_argument("--segment", default="attention", choices=["attention", "int32-int8"],
+                    help="attention: q/k/v in the cache dtype -> float output (the headline metric). "
+                         "int32-int8: the whole reference segment, int32 GEMM accumulators + scales in, "
+                         "per-token INT8 + scale out (implies --no-cpu)")
     args = ap.parse_args()
 
     if args.workload == "all":
@@ -150,8 +154,23 @@ def main() -> int:
 
     op = DecodeAttention(B, H, D, L, t_dt, nsplit=args.nsplit, device=dev)
     plan = op.plan(max_ctx, ragged)
+    extra = {}
+    if args.segment == "int32-int8":
+        # the segment as OpenDecoder::forward feeds it: int32 accumulators of the INT8 projections with
+        # activation/weight scales in, quantised attention output out
+        args.no_cpu = True
+        rng = np.random.default_rng(args.seed)
+        q, k, v = (torch.from_numpy(rng.integers(-20000, 20000, (B, 1, H, D), dtype=np.int32)).to(dev)
+                   for _ in range(3))
+        extra = dict(
+            qkv_inp_scale=torch.from_numpy(((rng.random(B) + 0.5) * 2e-3).astype(np.float32)).to(dev),
+            q_weight_scale=torch.from_numpy((rng.random(H * D) * 3e-2 + 1e-3).astype(np.float32)).to(dev),
+            k_weight_scale=torch.from_numpy((rng.random(H * D) * 3e-2 + 1e-3).astype(np.float32)).to(dev),
+            v_weight_scale=torch.from_numpy((rng.random(H * D) * 3e-2 + 1e-3).astype(np.float32)).to(dev),
+            out_int8=torch.empty(B, H * D, dtype=torch.int8, device=dev),
+            out_scale=torch.empty(B, dtype=torch.float32, device=dev))
     ios = [op.make_io(q, k, v, kc, vc, freq, out, start_pos=start_pos, start_pos_per_seq=pos_d,
-                      max_start_pos=start_pos if ragged else -1) for kc, vc in caches]
+                      max_start_pos=start_pos if ragged else -1, **extra) for kc, vc in caches]
     stream = torch.cuda.current_stream(dev)
 
     def run(n, passes=3):
@@ -247,6 +266,7 @@ def main() -> int:
             "sum_ctx": sum_ctx, "cache_rows": L, "cache_copies_rotated": copies,
             "nsplit": plan.nsplit, "chunk_rows": plan.chunk_rows, "two_pass": bool(plan.two_pass),
             "algorithmic_bytes_per_step": alg,
+            "segment": args.segment,
         },
         "roofline": {
             "bound": "hbm", "achieved": round(kern_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",

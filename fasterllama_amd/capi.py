@@ -33,6 +33,8 @@ EXPORTED_SYMBOLS = (
     "fl_decode_attn_plan",
     "fl_decode_attn_forward",
     "fl_decode_attn_forward_passes",
+    "fl_prefill_attn_workspace_bytes",
+    "fl_prefill_attn_forward",
     "fl_rope_table",
     "fl_kv_cache_bytes",
     "fl_attn_strerror",
@@ -119,6 +121,10 @@ def load() -> C.CDLL:
     lib.fl_decode_attn_forward.restype = C.c_int
     lib.fl_decode_attn_forward_passes.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnIO), C.c_void_p, C.c_int]
     lib.fl_decode_attn_forward_passes.restype = C.c_int
+    lib.fl_prefill_attn_workspace_bytes.argtypes = [C.POINTER(AttnDesc), C.c_int32, C.POINTER(C.c_size_t)]
+    lib.fl_prefill_attn_workspace_bytes.restype = C.c_int
+    lib.fl_prefill_attn_forward.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnIO), C.c_int32, C.c_void_p]
+    lib.fl_prefill_attn_forward.restype = C.c_int
     lib.fl_rope_table.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_float, C.c_void_p]
     lib.fl_rope_table.restype = C.c_int
     lib.fl_attn_strerror.argtypes = [C.c_int]

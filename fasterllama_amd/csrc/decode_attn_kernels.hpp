@@ -570,32 +570,6 @@ __global__ __launch_bounds__(kCombineThreads) void decode_attn_combine_kernel(co
     }
 }
 
-// grid = B, block = 1024.  Per-row absmax INT8 quantisation of the attention output of one sequence
-// (launchAttnQuantizedTransposeKernel, decoder_kernels.cu:1179-1212 with seq_len == 1):
-//   absmax = max(-1e9, max |x|); scale[b] = absmax/127; q = sat_s8(rint(x*127/absmax)).
-// The float output [B, H*D] was written by the streaming or the combine kernel.
-__global__ __launch_bounds__(1024) void attn_quantize_kernel(const float *__restrict__ attn, int8_t *__restrict__ out_q,
-                                                             float *__restrict__ out_scale, int HD)
-{
-    __shared__ float s_red[16];
-    const int b = blockIdx.x, tid = threadIdx.x;
-    const float *x = attn + (size_t)b * HD;
-    float absmax = kMaxFloor;
-    for (int e = tid; e < HD; e += 1024) absmax = fmaxf(absmax, fabsf(x[e]));
-    absmax = wave_max(absmax);
-    if ((tid & 63) == 0) s_red[tid >> 6] = absmax;
-    __syncthreads();
-    absmax = s_red[0];
-#pragma unroll
-    for (int w = 1; w < 16; ++w) absmax = fmaxf(absmax, s_red[w]);
-    if (tid == 0) out_scale[b] = absmax / 127.0f;
-    for (int e = tid; e < HD; e += 1024) {
-        const float v = rintf(__fmul_rn(x[e], 127.0f) / absmax);
-        const int qv = (v != v) ? 0 : (int)fminf(fmaxf(v, -128.f), 127.f); // NaN -> 0, saturate
-        out_q[(size_t)b * HD + e] = (int8_t)qv;
-    }
-}
-
 // ---------------------------------------------------------------- RoPE table producer
 
 // freq_cis[r, 2i] = cos(r * base^(-2i/D)), freq_cis[r, 2i+1] = sin(same); evaluated in double

@@ -9,6 +9,7 @@
 
 #include "../../include/fl_decode_attn.h"
 #include "decode_attn_kernels.hpp"
+#include "prefill_attn_kernels.hpp"
 
 namespace {
 
@@ -240,6 +241,55 @@ hipError_t dispatch_split(int D, const Params &p, dim3 grid, hipStream_t stream)
     }
 }
 
+// ---- prompt phase helpers
+
+bool prefill_head_dim_ok(int D) { return D == 32 || D == 64 || D == 128; }
+
+struct PrefillWorkspace {
+    size_t q_rot, tmp_out, total;
+};
+
+PrefillWorkspace prefill_workspace(const fl_attn_desc *d, int S)
+{
+    const size_t n = align_up((size_t)d->batch_size * d->head_num * (size_t)S * d->size_per_head * sizeof(float), 256);
+    PrefillWorkspace w;
+    w.q_rot = 0;
+    w.tmp_out = n;
+    w.total = 2 * n;
+    return w;
+}
+
+template <typename T, int D>
+hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
+{
+    constexpr int VEC = flattn::Vec16<T>::N;
+    constexpr int LPR = D / VEC < 64 ? D / VEC : 64;
+    constexpr int ROWS = 256 / LPR;
+    const int64_t rows = (int64_t)p.B * p.S * p.H;
+    hipLaunchKernelGGL((flattn::prefill_rope_append_kernel<T, D>), dim3((unsigned)((rows + ROWS - 1) / ROWS)), dim3(256), 0,
+                       stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const unsigned qblocks = (unsigned)((p.S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock);
+    const dim3 grid(qblocks * (unsigned)(p.B * p.H)); // (b,h) fastest: the query blocks of one head share an XCD's L2
+    if (p.attn_mask)
+        hipLaunchKernelGGL((flattn::prefill_attn_kernel<T, D, true>), grid, dim3(256), 0, stream, p);
+    else
+        hipLaunchKernelGGL((flattn::prefill_attn_kernel<T, D, false>), grid, dim3(256), 0, stream, p);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t dispatch_prefill(int D, const flattn::PrefillParams &p, hipStream_t stream)
+{
+    switch (D) {
+    case 32: return launch_prefill<T, 32>(p, stream);
+    case 64: return launch_prefill<T, 64>(p, stream);
+    case 128: return launch_prefill<T, 128>(p, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 } // namespace
@@ -375,8 +425,8 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
     if (passes & 2) {
         if (!direct && !check_hip(dispatch_combine(D, p, bh, stream))) return FL_ATTN_ERR_HIP;
         if (quant) {
-            hipLaunchKernelGGL(flattn::attn_quantize_kernel, dim3(desc->batch_size), dim3(1024), 0, stream, p.out,
-                               io->out_int8, io->out_scale, desc->head_num * D);
+            hipLaunchKernelGGL(flattn::attn_quantize_transpose_kernel, dim3(desc->batch_size), dim3(1024), 0, stream,
+                               p.out, io->out_int8, io->out_scale, desc->head_num, 1, D);
             if (!check_hip(hipGetLastError())) return FL_ATTN_ERR_HIP;
         }
     }
@@ -386,6 +436,74 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
 int fl_decode_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream)
 {
     return fl_decode_attn_forward_passes(desc, io, hip_stream, 3);
+}
+
+// ---- prompt phase --------------------------------------------------------------------------------
+
+int fl_prefill_attn_workspace_bytes(const fl_attn_desc *desc, int32_t seq_len, size_t *bytes)
+{
+    if (!bytes) return FL_ATTN_ERR_NULL_POINTER;
+    int st = validate_desc(desc);
+    if (st != FL_ATTN_OK) return st;
+    if (!prefill_head_dim_ok(desc->size_per_head)) return FL_ATTN_ERR_HEAD_DIM;
+    if (seq_len < 1 || seq_len > desc->total_len) return FL_ATTN_ERR_POSITION;
+    *bytes = prefill_workspace(desc, seq_len).total;
+    return FL_ATTN_OK;
+}
+
+int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int32_t seq_len, void *hip_stream)
+{
+    int st = validate_desc(desc);
+    if (st != FL_ATTN_OK) return st;
+    if (!prefill_head_dim_ok(desc->size_per_head)) return FL_ATTN_ERR_HEAD_DIM;
+    if (!io) return FL_ATTN_ERR_NULL_POINTER;
+    if (!io->q || !io->k_new || !io->v_new || !io->k_cache || !io->v_cache || !io->freq_cis)
+        return FL_ATTN_ERR_NULL_POINTER;
+    const bool quant = io->out_int8 != nullptr;
+    if (!io->out && !quant) return FL_ATTN_ERR_NULL_POINTER;
+    if (quant && !io->out_scale) return FL_ATTN_ERR_NULL_POINTER;
+    if (io->reserved != 0 || io->start_pos_per_seq) return FL_ATTN_ERR_ARGUMENT; // uniform positions only
+    const bool i32 = io->qkv_inp_scale != nullptr;
+    if (i32 && (!io->q_weight_scale || !io->k_weight_scale || !io->v_weight_scale)) return FL_ATTN_ERR_NULL_POINTER;
+    if (!i32 && (io->q_weight_scale || io->k_weight_scale || io->v_weight_scale)) return FL_ATTN_ERR_ARGUMENT;
+    if (!aligned16(io->q) || !aligned16(io->k_new) || !aligned16(io->v_new) || !aligned16(io->k_cache) ||
+        !aligned16(io->v_cache) || !aligned16(io->freq_cis) || !aligned16(io->out) ||
+        (i32 && (!aligned16(io->q_weight_scale) || !aligned16(io->k_weight_scale) || !aligned16(io->v_weight_scale))))
+        return FL_ATTN_ERR_ALIGNMENT;
+    const int L = desc->total_len;
+    if (seq_len < 1 || io->start_pos < 0 || (int64_t)io->start_pos + seq_len > L) return FL_ATTN_ERR_POSITION;
+    if (io->rope_row < FL_ATTN_ROPE_AT_POSITION) return FL_ATTN_ERR_POSITION;
+    if (io->attn_mask && io->mask_ld < 0) return FL_ATTN_ERR_ARGUMENT;
+    if ((int64_t)desc->batch_size * desc->head_num * ((seq_len + 127) / 128) > (int64_t)INT32_MAX) return FL_ATTN_ERR_SHAPE;
+
+    const PrefillWorkspace wl = prefill_workspace(desc, seq_len);
+    if (!io->workspace || io->workspace_bytes < wl.total) return FL_ATTN_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(io->workspace) & 255u) != 0) return FL_ATTN_ERR_WORKSPACE;
+    char *ws = static_cast<char *>(io->workspace);
+
+    const int D = desc->size_per_head;
+    flattn::PrefillParams p{};
+    p.q = io->q; p.k_new = io->k_new; p.v_new = io->v_new;
+    p.k_cache = io->k_cache; p.v_cache = io->v_cache;
+    p.freq_cis = io->freq_cis; p.attn_mask = io->attn_mask;
+    p.q_rot = reinterpret_cast<float *>(ws + wl.q_rot);
+    p.out = io->out ? io->out : reinterpret_cast<float *>(ws + wl.tmp_out);
+    p.inp_scale = io->qkv_inp_scale; p.wq_scale = io->q_weight_scale;
+    p.wk_scale = io->k_weight_scale; p.wv_scale = io->v_weight_scale;
+    p.mask_ld = io->mask_ld;
+    p.B = desc->batch_size; p.H = desc->head_num; p.L = L; p.S = seq_len;
+    p.start_pos = io->start_pos; p.rope_row = io->rope_row;
+    p.scale = desc->softmax_scale > 0.f ? desc->softmax_scale : 1.0f / sqrtf((float)D);
+
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    hipError_t e = desc->dtype == FL_ATTN_F16 ? dispatch_prefill<_Float16>(D, p, stream) : dispatch_prefill<float>(D, p, stream);
+    if (!check_hip(e)) return FL_ATTN_ERR_HIP;
+    if (quant) {
+        hipLaunchKernelGGL(flattn::attn_quantize_transpose_kernel, dim3((unsigned)(desc->batch_size * seq_len)), dim3(1024), 0,
+                           stream, p.out, io->out_int8, io->out_scale, desc->head_num, seq_len, D);
+        if (!check_hip(hipGetLastError())) return FL_ATTN_ERR_HIP;
+    }
+    return FL_ATTN_OK;
 }
 
 int fl_rope_table(float *freq_cis, int32_t rows, int32_t size_per_head, float base, void *hip_stream)

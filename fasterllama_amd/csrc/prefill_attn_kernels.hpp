@@ -1,0 +1,282 @@
+// Prompt-phase (seq_len > 1) self-attention for gfx950: the dense branch of the same block of
+// FasterLLaMA's OpenDecoder::forward (fasterLlama/cuda/open_decoder.cu:138-191, :207-228):
+//   RoPE + transpose + cache append     decoder_kernels.cu:425-464, :597-632, :858-884
+//   scores = Q K^T  (cublasGemmStridedBatchedEx, open_decoder.cu:181-190)
+//   block softmax with mask row start_pos + q  (decoder_kernels.cu:800-835)
+//   out = P V       (cublasGemmStridedBatchedEx, open_decoder.cu:218-227)
+// Unlike the decode step this is a dense contraction (S x ctx x D per head), so it runs on the
+// matrix cores: FP32 MFMA (v_mfma_f32_32x32x2_f32) with FP32 operands, which keeps the 1e-5
+// parity bar of the FP32 path; fp16 caches are widened to FP32 when a tile is staged in LDS.
+//
+// Two kernels:
+//   prefill_rope_append_kernel  elementwise: RoPE(q) -> workspace [B,H,S,D] fp32, RoPE(k), v ->
+//                               cache rows start_pos + s (bit-identical to the decode step's rows)
+//   prefill_attn_kernel         flash-attention style: a workgroup owns 128 queries of one (b,h)
+//                               (32 per wave) and walks the keys 32 at a time through LDS.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "decode_attn_kernels.hpp"
+
+namespace flattn {
+
+struct PrefillParams {
+    const void *q, *k_new, *v_new; // [B,S,H,D] storage dtype, or int32 accumulators
+    void *k_cache, *v_cache;       // [B,H,L,D]
+    const float *freq_cis;
+    const float *attn_mask;
+    float *q_rot; // workspace [B,H,S,D] fp32
+    float *out;   // [B,H,S,D] fp32
+    const float *inp_scale, *wq_scale, *wk_scale, *wv_scale;
+    int64_t mask_ld;
+    int32_t B, H, L, S;
+    int32_t start_pos, rope_row;
+    float scale;
+};
+
+// ---------------------------------------------------------------- RoPE + transpose + append
+
+// One lane-group (LPR lanes) per token-head row; grid covers B*S*H rows, 256 threads per block.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillParams p)
+{
+    typedef typename Vec16<T>::type V;
+    constexpr int VEC = Vec16<T>::N;
+    constexpr int CH = D / VEC;
+    constexpr int LPR = CH < 64 ? CH : 64;
+    constexpr int CPL = CH / LPR;
+    constexpr int ROWS = 256 / LPR;
+
+    const int64_t rows = (int64_t)p.B * p.S * p.H;
+    const int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / LPR; // index into [B,S,H]
+    if (row >= rows) return;
+    const int lig = threadIdx.x % LPR;
+    const int h = (int)(row % p.H);
+    const int64_t bs = row / p.H;
+    const int s = (int)(bs % p.S), b = (int)(bs / p.S);
+    const int pos = p.start_pos + s;
+    const int rope_row = p.rope_row < 0 ? pos : p.rope_row + s;
+    const float *freq = p.freq_cis + (size_t)rope_row * D;
+    const bool is_i32 = p.inp_scale != nullptr;
+    const float inp_scale = is_i32 ? p.inp_scale[bs] : 0.f;
+    const size_t in_off = (size_t)row * D;
+    const size_t bh = (size_t)b * p.H + h;
+    float *qdst = p.q_rot + (bh * p.S + s) * D;
+    T *kdst = reinterpret_cast<T *>(p.k_cache) + (bh * p.L + pos) * D;
+    T *vdst = reinterpret_cast<T *>(p.v_cache) + (bh * p.L + pos) * D;
+
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+        const int e0 = (c * LPR + lig) * VEC;
+        float qx[VEC], kx[VEC], vx[VEC];
+        load_token_chunk<T, VEC>(p.q, in_off + e0, is_i32, inp_scale, is_i32 ? p.wq_scale + h * D + e0 : nullptr, qx);
+        load_token_chunk<T, VEC>(p.k_new, in_off + e0, is_i32, inp_scale, is_i32 ? p.wk_scale + h * D + e0 : nullptr, kx);
+        load_token_chunk<T, VEC>(p.v_new, in_off + e0, is_i32, inp_scale, is_i32 ? p.wv_scale + h * D + e0 : nullptr, vx);
+        V kt, vt;
+#pragma unroll
+        for (int i = 0; i < VEC; i += 4) {
+            const float4 f = *reinterpret_cast<const float4 *>(freq + e0 + i);
+            float4 qo;
+            rope_pair(qx[i], qx[i + 1], f.x, f.y, qo.x, qo.y);
+            rope_pair(qx[i + 2], qx[i + 3], f.z, f.w, qo.z, qo.w);
+            *reinterpret_cast<float4 *>(qdst + e0 + i) = qo;
+            float r0, r1, r2, r3;
+            rope_pair(kx[i], kx[i + 1], f.x, f.y, r0, r1);
+            rope_pair(kx[i + 2], kx[i + 3], f.z, f.w, r2, r3);
+            kt[i] = to_storage<T>(r0); kt[i + 1] = to_storage<T>(r1);
+            kt[i + 2] = to_storage<T>(r2); kt[i + 3] = to_storage<T>(r3);
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) vt[i] = to_storage<T>(vx[i]);
+        *reinterpret_cast<V *>(kdst + e0) = kt;
+        *reinterpret_cast<V *>(vdst + e0) = vt;
+    }
+}
+
+// ---------------------------------------------------------------- dense attention on MFMA
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kPrefillQueriesPerBlock = 128; // 4 waves x 32 queries
+constexpr int kPrefillKeysPerStep = 32;
+
+// MFMA operand layouts used below (v_mfma_f32_32x32x2_f32, D += A(32x2) * B(2x32)):
+//   A: lane holds A[row = lane % 32][k = lane / 32];  B: lane holds B[k = lane / 32][col = lane % 32];
+//   D: register v of a lane holds D[row = 8*(v/4) + 4*(lane/32) + (v%4)][col = lane % 32].
+// Scores are formed transposed, S^T = K Q^T (rows = keys, cols = queries), so a lane ends up with
+// 16 probabilities of ONE query — exactly the B operand of the second product O^T = V^T P^T:
+// no LDS transpose of P, and the softmax row reductions are in-lane plus one cross-half exchange.
+// The contraction index of the first product is enumerated as d = 8c + 4*(lane/32) + r
+// (c = chunk, r = 0..3) so that each lane fetches its K operand as one 128-bit LDS read.
+template <typename T, int D, bool HAS_MASK>
+__global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p)
+{
+    typedef typename Vec16<T>::type V;
+    constexpr int VEC = Vec16<T>::N;
+    constexpr int BN = kPrefillKeysPerStep;
+    constexpr int LDK = D + 4; // padded LDS row (floats): rows start 4 banks apart
+    constexpr int NC = D / 8;
+    constexpr int NDT = D / 32;
+    constexpr int CPR = D / VEC; // 16-byte chunks per cache row
+    static_assert(D % 32 == 0, "head size must be a multiple of 32");
+
+    __shared__ float sK[BN][LDK];
+    __shared__ float sV[BN][LDK];
+
+    const int BH = p.B * p.H;
+    const int qb = blockIdx.x / BH, bh = blockIdx.x % BH;
+    const int S = p.S, P = p.start_pos, L = p.L;
+    const int ctx = P + S;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int qi = lane & 31, hf = lane >> 5;
+    const int q_row = qb * kPrefillQueriesPerBlock + wave * 32 + qi;
+    const bool q_ok = q_row < S;
+
+    float qreg[NC][4];
+    {
+        const float *qsrc = p.q_rot + ((size_t)bh * S + (q_ok ? q_row : 0)) * D + 4 * hf;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            float4 t = q_ok ? *reinterpret_cast<const float4 *>(qsrc + 8 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
+            qreg[c][0] = t.x; qreg[c][1] = t.y; qreg[c][2] = t.z; qreg[c][3] = t.w;
+        }
+    }
+
+    floatx16 ot[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) ot[dt][v] = 0.f;
+    float m = kMaxFloor, l = 0.f;
+    const float *mrow = HAS_MASK ? p.attn_mask + (size_t)(P + (q_ok ? q_row : 0)) * p.mask_ld : nullptr;
+    const T *Kb = reinterpret_cast<const T *>(p.k_cache) + (size_t)bh * L * D;
+    const T *Vb = reinterpret_cast<const T *>(p.v_cache) + (size_t)bh * L * D;
+    const float scale = p.scale;
+
+    for (int k0 = 0; k0 < ctx; k0 += BN) {
+        __syncthreads(); // every wave is done with the previous tile
+        for (int idx = tid; idx < BN * CPR; idx += 256) {
+            const int r = idx / CPR, cc = idx % CPR;
+            const int key = k0 + r;
+            float kf[VEC], vf[VEC];
+            if (key < ctx) {
+                const V kx = *reinterpret_cast<const V *>(Kb + (size_t)key * D + cc * VEC);
+                const V vx = *reinterpret_cast<const V *>(Vb + (size_t)key * D + cc * VEC);
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) { kf[i] = (float)kx[i]; vf[i] = (float)vx[i]; }
+            } else { // past the context: zeros, and the scores are forced to -inf below
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) { kf[i] = 0.f; vf[i] = 0.f; }
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; i += 4) {
+                *reinterpret_cast<float4 *>(&sK[r][cc * VEC + i]) = make_float4(kf[i], kf[i + 1], kf[i + 2], kf[i + 3]);
+                *reinterpret_cast<float4 *>(&sV[r][cc * VEC + i]) = make_float4(vf[i], vf[i + 1], vf[i + 2], vf[i + 3]);
+            }
+        }
+        float mk[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int key = k0 + 8 * (v / 4) + 4 * hf + (v % 4);
+            mk[v] = (HAS_MASK && key < ctx) ? mrow[key] : 0.f;
+        }
+        __syncthreads();
+
+        // S^T tile: 32 keys x 32 queries, contraction over D
+        floatx16 st;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) st[v] = 0.f;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const float4 ka = *reinterpret_cast<const float4 *>(&sK[qi][8 * c + 4 * hf]);
+            st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.x, qreg[c][0], st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.y, qreg[c][1], st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.z, qreg[c][2], st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.w, qreg[c][3], st, 0, 0, 0);
+        }
+
+        // softmax update of this lane's query: v = s*scale + mask, floor -1e9 (decoder_kernels.cu:811-820)
+        float sc[16];
+        float mx = m;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int key = k0 + 8 * (v / 4) + 4 * hf + (v % 4);
+            float x = HAS_MASK ? fmaf(st[v], scale, mk[v]) : st[v] * scale;
+            if (key >= ctx) x = -__builtin_inff();
+            sc[v] = x;
+            mx = fmaxf(mx, x);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32)); // the other half-wave holds the other 16 keys of this query
+        const float alpha = expf(m - mx);
+        m = mx;
+        l *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) ot[dt][v] *= alpha;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            sc[v] = expf(sc[v] - m);
+            l += sc[v];
+        }
+
+        // O^T += V^T P^T: contraction over the 32 keys, two per MFMA (key of step t in half hf:
+        // 8*(t/4) + 4*hf + (t%4), the key whose probability this lane holds in sc[t])
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int t = 0; t < 16; ++t) {
+                const float va = sV[8 * (t / 4) + 4 * hf + (t % 4)][32 * dt + qi];
+                ot[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(va, sc[t], ot[dt], 0, 0, 0);
+            }
+    }
+
+    l += __shfl_xor(l, 32);
+    if (q_ok) {
+        float *dst = p.out + ((size_t)bh * S + q_row) * D;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                float4 r;
+                r.x = ot[dt][4 * g4 + 0] / l; // p = e / sum (decoder_kernels.cu:833)
+                r.y = ot[dt][4 * g4 + 1] / l;
+                r.z = ot[dt][4 * g4 + 2] / l;
+                r.w = ot[dt][4 * g4 + 3] / l;
+                *reinterpret_cast<float4 *>(dst + 32 * dt + 8 * g4 + 4 * hf) = r;
+            }
+    }
+}
+
+// ---------------------------------------------------------------- INT8 epilogue with transpose
+
+// grid = B*S, block = 1024.  attn [B,H,S,D] float -> out_q [B,S,H*D] int8, out_scale [B,S]
+// (launchAttnQuantizedTransposeKernel, decoder_kernels.cu:1179-1255); S == 1 is the decode case.
+__global__ __launch_bounds__(1024) void attn_quantize_transpose_kernel(const float *__restrict__ attn,
+                                                                       int8_t *__restrict__ out_q,
+                                                                       float *__restrict__ out_scale, int H, int S, int D)
+{
+    __shared__ float s_red[16];
+    const int bs = blockIdx.x, tid = threadIdx.x;
+    const int b = bs / S, s = bs % S;
+    const int HD = H * D;
+    const float *x = attn + ((size_t)b * H * S + s) * D; // + h * S * D + d
+    float absmax = kMaxFloor;
+    for (int e = tid; e < HD; e += 1024) absmax = fmaxf(absmax, fabsf(x[(size_t)(e / D) * S * D + e % D]));
+    absmax = wave_max(absmax);
+    if ((tid & 63) == 0) s_red[tid >> 6] = absmax;
+    __syncthreads();
+    absmax = s_red[0];
+#pragma unroll
+    for (int w = 1; w < 16; ++w) absmax = fmaxf(absmax, s_red[w]);
+    if (tid == 0) out_scale[bs] = absmax / 127.0f;
+    for (int e = tid; e < HD; e += 1024) {
+        const float v = rintf(__fmul_rn(x[(size_t)(e / D) * S * D + e % D], 127.0f) / absmax);
+        const int qv = (v != v) ? 0 : (int)fminf(fmaxf(v, -128.f), 127.f); // NaN -> 0, saturate
+        out_q[(size_t)bs * HD + e] = (int8_t)qv;
+    }
+}
+
+} // namespace flattn

@@ -96,6 +96,40 @@ class DecodeAttention:
         return out
 
 
+class PrefillAttention(DecodeAttention):
+    """Prompt-phase attention (seq_len new tokens per sequence) over the same caller-owned caches.
+
+    q/k_new/v_new are [B, seq_len, H, D]; the result is [B, H, seq_len, D] float32, the layout of the
+    reference's qkv_buf_ (open_decoder.h:61)."""
+
+    def __init__(self, batch_size: int, head_num: int, size_per_head: int, total_len: int, max_seq_len: int,
+                 dtype: torch.dtype = torch.float16, softmax_scale: float = 0.0,
+                 device: str | torch.device = "cuda:0"):
+        super().__init__(batch_size, head_num, size_per_head, total_len, dtype, 0, softmax_scale, device)
+        n = C.c_size_t(0)
+        capi.check(self.lib.fl_prefill_attn_workspace_bytes(C.byref(self.desc), max_seq_len, C.byref(n)))
+        self.max_seq_len = max_seq_len
+        self.workspace = torch.empty(max(n.value, self.workspace.numel()), dtype=torch.uint8, device=self.device)
+
+    def launch_prefill(self, io: capi.AttnIO, seq_len: int, stream: torch.cuda.Stream | None = None) -> int:
+        s = stream if stream is not None else torch.cuda.current_stream(self.device)
+        with torch.cuda.device(self.device):
+            return self.lib.fl_prefill_attn_forward(C.byref(self.desc), C.byref(io), seq_len,
+                                                    C.c_void_p(s.cuda_stream))
+
+    def prefill(self, q, k_new, v_new, k_cache, v_cache, freq_cis, start_pos: int = 0, out=None, **kw):
+        d = self.desc
+        seq_len = q.shape[1]
+        if seq_len > self.max_seq_len:
+            raise capi.FlAttnError(capi.FL_ATTN_ERR_WORKSPACE, "seq_len exceeds the workspace this object was sized for")
+        if out is None and kw.get("out_int8") is None:
+            out = torch.empty(d.batch_size, d.head_num, seq_len, d.size_per_head, dtype=torch.float32,
+                              device=self.device)
+        io = self.make_io(q, k_new, v_new, k_cache, v_cache, freq_cis, out, start_pos=start_pos, **kw)
+        capi.check(self.launch_prefill(io, seq_len))
+        return out
+
+
 def rope_table(rows: int, size_per_head: int, base: float = 10000.0,
                device: str | torch.device = "cuda:0") -> torch.Tensor:
     """Device RoPE table [rows, D] (replaces launchPrecomputeFreqsCis, decoding_kernels.cu:116-135)."""

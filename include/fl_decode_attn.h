@@ -129,6 +129,22 @@ int fl_decode_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, void 
 int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream,
                                   int passes);
 
+/* ---- prompt phase (seq_len > 1): the dense branch of the same block -------------------------------
+ * Replaces, for seq_len new tokens per sequence at positions start_pos .. start_pos+seq_len-1
+ * (open_decoder.cu:138-191, :207-228, :245-246):
+ *   launchQKRoteEmbeddingTranspose / launchDequantizedVTransposeKernel / launchStoreKVcacheKernel,
+ *   cublasGemmStridedBatchedEx (Q K^T, :181-190), launchBlockSoftmaxKernel (:207-208),
+ *   cublasGemmStridedBatchedEx (P V, :218-227), launchAttnQuantizedTransposeKernel (:245-246).
+ * fl_attn_io is read as follows: q/k_new/v_new are [B, seq_len, H, D] (cache dtype, or int32
+ * accumulators with qkv_inp_scale [B, seq_len]); out is [B, H, seq_len, D] float (open_decoder.h:61);
+ * out_int8 is [B, seq_len, H*D] with out_scale [B, seq_len]; query s uses mask row start_pos + s and
+ * RoPE table row start_pos + s (rope_row == FL_ATTN_ROPE_AT_POSITION) or rope_row + s;
+ * start_pos_per_seq must be NULL.  Keys are the cache rows [0, start_pos + seq_len) after the append.
+ * size_per_head must be 32, 64 or 128.  Workspace: fl_prefill_attn_workspace_bytes(). */
+int fl_prefill_attn_workspace_bytes(const fl_attn_desc *desc, int32_t seq_len, size_t *bytes);
+int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int32_t seq_len,
+                            void *hip_stream);
+
 /* RoPE table producer on the device: rows x D floats, row r = [cos(r*w_0), sin(r*w_0), ...],
  * w_i = base^(-2i/D).  Replaces launchPrecomputeFreqsCis (decoding_kernels.cu:85-135,
  * called at decoding_sampling.cu:190) with correctly rounded sincos instead of fast intrinsics. */

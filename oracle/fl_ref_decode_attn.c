@@ -374,6 +374,215 @@ int fl_ref_decode_attn_i32(int dtype, int B, int H, int D, int L, const int32_t 
     return run(&a, threads);
 }
 
+/* ------------------------------------------------------------------ the prompt phase (seq_len > 1)
+ *
+ * Restates the seq_len > 1 branch of the same block (open_decoder.cu:138-191, :207-228):
+ *   RoPE of every new token with table row (position of the token) (decoder_kernels.cu:440, :455-458),
+ *   transpose [B,S,H,D] -> [B,H,S,D] (:461), append at cache rows start_pos + s (:605-610),
+ *   scores = Q K^T (open_decoder.cu:181-190), softmax row q with mask row start_pos + q
+ *   (decoder_kernels.cu:806-833 with mask_offset = seq_q_id * max_seq_len on top of the
+ *   start_pos * total_len_ offset of open_decoder.cu:207), out = P V (open_decoder.cu:218-227),
+ *   output layout [B,H,S,D] (open_decoder.h:61).
+ * The reference multiplies by the NEW keys only (key_out_buf_), which equals the cache rows
+ * [0, S) because its driver always calls the prompt phase with start_pos == 0
+ * (decoding_sampling.cu:197-258).  This restatement attends over cache rows [0, start_pos + S),
+ * which is the same thing for start_pos == 0 and extends it to a chunked prompt otherwise.
+ * With S == 1 it performs exactly the operations of fl_ref_decode_attn, in the same order.
+ */
+static void prefill_one_head(const ref_args *a, int S, int b, int h, float *scratch)
+{
+    const int D = a->D, H = a->H, L = a->L, dt = a->dtype, P = a->start_pos;
+    const int ctx = P + S;
+    const size_t cache_row0 = ((size_t)b * H + h) * (size_t)L * D;
+    float *qr = scratch;                 /* S * D rotated queries */
+    float *sc = scratch + (size_t)S * D; /* ctx scores */
+
+    for (int s = 0; s < S; ++s) {
+        const int row = a->rope_row < 0 ? P + s : a->rope_row + s;
+        const float *f = a->freq_cis + (size_t)row * D;
+        const size_t in_off = (((size_t)b * S + s) * H + h) * D; /* [B,S,H,D] */
+        const size_t new_off = cache_row0 + (size_t)(P + s) * D;
+        for (int i = 0; i < D; i += 2) {
+            float q0, q1, k0, k1, v0, v1;
+            if (a->inp_scale) {
+                const int32_t *qi = (const int32_t *)a->q, *ki = (const int32_t *)a->k_new,
+                              *vi = (const int32_t *)a->v_new;
+                float sc_in = a->inp_scale[(size_t)b * S + s]; /* [B,S] */
+                q0 = dequant(qi[in_off + i], sc_in, a->wq_scale[h * D + i]);
+                q1 = dequant(qi[in_off + i + 1], sc_in, a->wq_scale[h * D + i + 1]);
+                k0 = dequant(ki[in_off + i], sc_in, a->wk_scale[h * D + i]);
+                k1 = dequant(ki[in_off + i + 1], sc_in, a->wk_scale[h * D + i + 1]);
+                v0 = dequant(vi[in_off + i], sc_in, a->wv_scale[h * D + i]);
+                v1 = dequant(vi[in_off + i + 1], sc_in, a->wv_scale[h * D + i + 1]);
+            } else {
+                q0 = load_elem(a->q, in_off + i, dt);
+                q1 = load_elem(a->q, in_off + i + 1, dt);
+                k0 = load_elem(a->k_new, in_off + i, dt);
+                k1 = load_elem(a->k_new, in_off + i + 1, dt);
+                v0 = load_elem(a->v_new, in_off + i, dt);
+                v1 = load_elem(a->v_new, in_off + i + 1, dt);
+            }
+            float c = f[i], sn = f[i + 1], r0, r1;
+            rope_pair(q0, q1, c, sn, &qr[(size_t)s * D + i], &qr[(size_t)s * D + i + 1]);
+            rope_pair(k0, k1, c, sn, &r0, &r1);
+            store_elem(a->k_cache, new_off + i, dt, r0);
+            store_elem(a->k_cache, new_off + i + 1, dt, r1);
+            store_elem(a->v_cache, new_off + i, dt, v0);
+            store_elem(a->v_cache, new_off + i + 1, dt, v1);
+        }
+    }
+
+    for (int s = 0; s < S; ++s) {
+        const float *q = qr + (size_t)s * D;
+        float *o_row = a->out + ((((size_t)b * H + h) * S) + s) * D; /* [B,H,S,D] */
+        const float *mrow = a->attn_mask ? a->attn_mask + (size_t)(P + s) * (size_t)a->mask_ld : NULL;
+        if (!a->acc_double) {
+            float m = -1e9f;
+            for (int j = 0; j < ctx; ++j) {
+                float acc = 0.0f;
+                const size_t r = cache_row0 + (size_t)j * D;
+                for (int d = 0; d < D; ++d)
+                    acc += load_elem(a->k_cache, r + d, dt) * q[d];
+                float v = acc * a->scale + (mrow ? mrow[j] : 0.0f);
+                sc[j] = v;
+                m = fmaxf(m, v);
+            }
+            float sum = 0.0f;
+            for (int j = 0; j < ctx; ++j) {
+                float e = expf(sc[j] - m);
+                sc[j] = e;
+                sum += e;
+            }
+            for (int j = 0; j < ctx; ++j)
+                sc[j] = sc[j] / sum;
+            for (int d = 0; d < D; ++d)
+                o_row[d] = 0.0f;
+            for (int j = 0; j < ctx; ++j) {
+                const size_t r = cache_row0 + (size_t)j * D;
+                const float p = sc[j];
+                for (int d = 0; d < D; ++d)
+                    o_row[d] += p * load_elem(a->v_cache, r + d, dt);
+            }
+        } else {
+            double *scd = (double *)(scratch + (size_t)S * D + ((ctx + 1) & ~1));
+            double m = -1e9;
+            for (int j = 0; j < ctx; ++j) {
+                double acc = 0.0;
+                const size_t r = cache_row0 + (size_t)j * D;
+                for (int d = 0; d < D; ++d)
+                    acc += (double)load_elem(a->k_cache, r + d, dt) * (double)q[d];
+                double v = acc * (double)a->scale + (mrow ? (double)mrow[j] : 0.0);
+                scd[j] = v;
+                if (v > m)
+                    m = v;
+            }
+            double sum = 0.0;
+            for (int j = 0; j < ctx; ++j) {
+                scd[j] = exp(scd[j] - m);
+                sum += scd[j];
+            }
+            for (int d = 0; d < D; ++d) {
+                double acc = 0.0;
+                for (int j = 0; j < ctx; ++j)
+                    acc += scd[j] * (double)load_elem(a->v_cache, cache_row0 + (size_t)j * D + d, dt);
+                o_row[d] = (float)(acc / sum);
+            }
+        }
+    }
+}
+
+/*
+ * Prompt-phase attention for S new tokens per sequence at positions start_pos .. start_pos+S-1.
+ * q/k_new/v_new: [B,S,H,D] in the storage dtype (or int32 accumulators when inp_scale != NULL, with
+ * inp_scale [B,S]); out: [B,H,S,D] float.  rope_row < 0: table row = token position; otherwise
+ * row = rope_row + s.
+ */
+int fl_ref_prefill_attn(int dtype, int B, int H, int D, int L, int S, const void *q, const void *k_new,
+                        const void *v_new, const float *inp_scale, const float *wq_scale,
+                        const float *wk_scale, const float *wv_scale, void *k_cache, void *v_cache,
+                        const float *freq_cis, int rope_row, const float *attn_mask, int64_t mask_ld,
+                        int start_pos, float scale, float *out, int acc_double, int threads)
+{
+    if (!q || !k_new || !v_new || !k_cache || !v_cache || !freq_cis || !out)
+        return -1;
+    if (B <= 0 || H <= 0 || D <= 0 || (D & 1) || L <= 0 || S <= 0)
+        return -3;
+    if (dtype != FL_REF_F32 && dtype != FL_REF_F16)
+        return -6;
+    if (start_pos < 0 || start_pos + S > L)
+        return -4;
+    if (inp_scale && (!wq_scale || !wk_scale || !wv_scale))
+        return -1;
+    ref_args a;
+    memset(&a, 0, sizeof a);
+    a.dtype = dtype; a.B = B; a.H = H; a.D = D; a.L = L;
+    a.q = q; a.k_new = k_new; a.v_new = v_new; a.k_cache = k_cache; a.v_cache = v_cache;
+    a.freq_cis = freq_cis; a.rope_row = rope_row; a.attn_mask = attn_mask; a.mask_ld = mask_ld;
+    a.start_pos = start_pos; a.scale = scale; a.out = out; a.acc_double = acc_double;
+    a.inp_scale = inp_scale; a.wq_scale = wq_scale; a.wk_scale = wk_scale; a.wv_scale = wv_scale;
+    const int BH = B * H;
+    const size_t per = (size_t)S * D + (size_t)L + 2 + 2 * ((size_t)L + 2);
+    if (threads < 1)
+        threads = 1;
+    int fail = 0;
+#ifdef _OPENMP
+#pragma omp parallel num_threads(threads)
+#endif
+    {
+        float *scratch = (float *)malloc(per * sizeof(float));
+        if (!scratch) {
+#ifdef _OPENMP
+#pragma omp atomic write
+#endif
+            fail = 1;
+        }
+#ifdef _OPENMP
+#pragma omp for schedule(dynamic, 1)
+#endif
+        for (int bh = 0; bh < BH; ++bh)
+            if (scratch)
+                prefill_one_head(&a, S, bh / H, bh % H, scratch);
+        free(scratch);
+    }
+    return fail ? -7 : 0;
+}
+
+/*
+ * Per-token absmax INT8 quantisation with the [B,H,S,D] -> [B,S,H*D] transpose of
+ * launchAttnQuantizedTransposeKernel (decoder_kernels.cu:1179-1255): one scale per (b, s) over the
+ * H*D values of that token.  attn: [B,H,S,D] float; out_q: [B,S,H*D] int8; out_scale: [B,S].
+ */
+int fl_ref_attn_quantize_transpose(int B, int H, int S, int D, const float *attn, int8_t *out_q,
+                                   float *out_scale)
+{
+    if (!attn || !out_q || !out_scale)
+        return -1;
+    for (int b = 0; b < B; ++b)
+        for (int s = 0; s < S; ++s) {
+            float absmax = -1e9f;
+            for (int h = 0; h < H; ++h)
+                for (int d = 0; d < D; ++d)
+                    absmax = fmaxf(absmax, fabsf(attn[(((size_t)b * H + h) * S + s) * D + d]));
+            out_scale[(size_t)b * S + s] = absmax / 127.0f;
+            for (int h = 0; h < H; ++h)
+                for (int d = 0; d < D; ++d) {
+                    float v = attn[(((size_t)b * H + h) * S + s) * D + d] * 127.0f / absmax;
+                    float r = nearbyintf(v);
+                    int8_t o;
+                    if (v != v)
+                        o = 0;
+                    else if (r > 127.0f)
+                        o = 127;
+                    else if (r < -128.0f)
+                        o = -128;
+                    else
+                        o = (int8_t)r;
+                    out_q[((size_t)b * S + s) * H * D + (size_t)h * D + d] = o;
+                }
+        }
+    return 0;
+}
+
 /*
  * Per-row absmax INT8 quantisation of the attention output
  * (decoder_kernels.cu:1179-1212 for seq_len == 1):

@@ -32,6 +32,14 @@ def load() -> C.CDLL:
         lib.fl_ref_freq_cis.restype = C.c_int
         lib.fl_ref_attn_quantize.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         lib.fl_ref_attn_quantize.restype = C.c_int
+        lib.fl_ref_prefill_attn.argtypes = [
+            C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+            C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int64,
+            C.c_int, C.c_float, C.c_void_p, C.c_int, C.c_int]
+        lib.fl_ref_prefill_attn.restype = C.c_int
+        lib.fl_ref_attn_quantize_transpose.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                                       C.c_void_p]
+        lib.fl_ref_attn_quantize_transpose.restype = C.c_int
         lib.fl_ref_half_to_float.argtypes = [C.c_uint16]
         lib.fl_ref_half_to_float.restype = C.c_float
         lib.fl_ref_float_to_half.argtypes = [C.c_float]
@@ -107,4 +115,44 @@ def attn_quantize(attn: np.ndarray):
     rc = load().fl_ref_attn_quantize(B, HD, attn.ctypes.data, q.ctypes.data, s.ctypes.data)
     if rc != 0:
         raise ValueError(f"fl_ref_attn_quantize -> {rc}")
+    return q, s
+
+
+def prefill_attn(q, k_new, v_new, k_cache, v_cache, freq, start_pos=0, rope_row=-1, attn_mask=None, mask_ld=None,
+                 scale=None, acc_double=False, threads=1, inp_scale=None, wq_scale=None, wk_scale=None,
+                 wv_scale=None):
+    """Prompt phase, IN PLACE on the caches.  q/k_new/v_new: [B,S,H,D]; returns out [B,H,S,D] float32."""
+    B, H, L, D = k_cache.shape
+    S = q.shape[1]
+    assert q.shape == (B, S, H, D) and k_new.shape == q.shape and v_new.shape == q.shape
+    st = np.dtype(k_cache.dtype)
+    code = {np.dtype(np.float32): 0, np.dtype(np.float16): 1}[st]
+    for a in (q, k_new, v_new, k_cache, v_cache, freq):
+        assert a.flags.c_contiguous
+    if inp_scale is None:
+        assert q.dtype == st
+    else:
+        assert q.dtype == np.int32 and inp_scale.size == B * S
+    if scale is None:
+        scale = float(np.float32(1.0) / np.sqrt(np.float32(D)))
+    if mask_ld is None:
+        mask_ld = L
+    out = np.empty((B, H, S, D), dtype=np.float32)
+    rc = load().fl_ref_prefill_attn(code, B, H, D, L, S, _p(q), _p(k_new), _p(v_new), _p(inp_scale), _p(wq_scale),
+                                    _p(wk_scale), _p(wv_scale), _p(k_cache), _p(v_cache), _p(freq), rope_row,
+                                    _p(attn_mask), mask_ld, start_pos, scale, _p(out), int(acc_double), threads)
+    if rc != 0:
+        raise ValueError(f"fl_ref_prefill_attn -> {rc}")
+    return out
+
+
+def attn_quantize_transpose(attn: np.ndarray):
+    """[B,H,S,D] float32 -> (int8 [B,S,H*D], scale [B,S])."""
+    attn = np.ascontiguousarray(attn, dtype=np.float32)
+    B, H, S, D = attn.shape
+    q = np.empty((B, S, H * D), dtype=np.int8)
+    s = np.empty((B, S), dtype=np.float32)
+    rc = load().fl_ref_attn_quantize_transpose(B, H, S, D, attn.ctypes.data, q.ctypes.data, s.ctypes.data)
+    if rc != 0:
+        raise ValueError(f"fl_ref_attn_quantize_transpose -> {rc}")
     return q, s

@@ -1,0 +1,178 @@
+"""Prompt-phase (seq_len > 1) attention through the C ABI against the CPU oracle."""
+import numpy as np
+import pytest
+
+from fasterllama_amd import capi, synth
+from helpers import assert_cache_bit_exact, assert_out_close
+from oracle import ref
+
+pytestmark = pytest.mark.gpu
+NP_DT = {"f32": np.float32, "f16": np.float16}
+
+
+def causal_mask(L, fill=-1e5):
+    return np.where(np.arange(L)[None, :] > np.arange(L)[:, None], fill, 0.0).astype(np.float32)
+
+
+def make(B, H, D, L, S, dtype, seed=11):
+    dt = NP_DT[dtype]
+    q = synth.normal((B, S, H, D), dt, synth.TENSOR_Q, seed)
+    k = synth.normal((B, S, H, D), dt, synth.TENSOR_K_NEW, seed)
+    v = synth.normal((B, S, H, D), dt, synth.TENSOR_V_NEW, seed)
+    kc = synth.normal((B, H, L, D), dt, synth.TENSOR_K_CACHE, seed)
+    vc = synth.normal((B, H, L, D), dt, synth.TENSOR_V_CACHE, seed)
+    return q, k, v, kc, vc, synth.freq_cis_table(L, D)
+
+
+def run_both(gpu, B, H, D, L, S, P, dtype, mask=None, rope_row=-1, pad_nan=True, seed=11):
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    q, k, v, kc, vc, f = make(B, H, D, L, S, dtype, seed)
+    if pad_nan:  # rows at and after the first new token are stale: they must never be read before being written
+        kc[:, :, P:, :] = np.nan
+        vc[:, :, P:, :] = np.nan
+    kc_ref, vc_ref = kc.copy(), vc.copy()
+    want = ref.prefill_attn(q, k, v, kc_ref, vc_ref, f, start_pos=P, rope_row=rope_row, attn_mask=mask,
+                            acc_double=True, threads=16)
+    t = lambda a: None if a is None else torch.from_numpy(a).to(gpu)
+    op = PrefillAttention(B, H, D, L, S, torch.float16 if dtype == "f16" else torch.float32, device=gpu)
+    kc_d, vc_d = t(kc), t(vc)
+    out = op.prefill(t(q), t(k), t(v), kc_d, vc_d, t(f), start_pos=P, rope_row=rope_row, attn_mask=t(mask))
+    torch.cuda.synchronize()
+    kc_g, vc_g = kc_d.cpu().numpy(), vc_d.cpu().numpy()
+    # rows past the prompt were NaN before and must still be: compare bit patterns of everything
+    assert_cache_bit_exact(kc_g, kc_ref, "k_cache")
+    assert_cache_bit_exact(vc_g, vc_ref, "v_cache")
+    return out.cpu().numpy(), want, op
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+@pytest.mark.parametrize("S,P", [(1, 0), (2, 0), (31, 0), (32, 0), (33, 0), (100, 0), (128, 0), (129, 0), (300, 0),
+                                 (50, 37), (1, 200), (64, 64)])
+def test_prefill_matches_oracle(gpu, dtype, S, P):
+    L = 512
+    out, want, _ = run_both(gpu, 2, 3, 128, L, S, P, dtype, mask=causal_mask(L), seed=S + P)
+    assert_out_close(out, want, dtype, f"S={S} P={P}")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+@pytest.mark.parametrize("D", [32, 64, 128])
+def test_prefill_head_sizes_and_no_mask(gpu, dtype, D):
+    out, want, _ = run_both(gpu, 2, 5, D, 256, 77, 10, dtype, mask=None, seed=D)
+    assert_out_close(out, want, dtype, f"D={D} no mask")
+
+
+def test_prefill_strict_mask_first_row_is_nan(gpu):
+    # the samples' strict mask hides every key of query 0 at position 0: 0/0 = NaN, as the reference arithmetic
+    L = 64
+    fm = np.finfo(np.float32).max
+    m = np.where(np.arange(L)[:, None] > np.arange(L)[None, :], 0.0, -fm).astype(np.float32)
+    out, want, _ = run_both(gpu, 1, 2, 64, L, 40, 0, "f32", mask=m)
+    assert np.isnan(want[:, :, 0]).all() and np.isnan(out[:, :, 0]).all()
+    assert_out_close(out[:, :, 1:], want[:, :, 1:], "f32", "strict mask rows 1..")
+
+
+def test_prefill_literal_rope_rows(gpu):
+    # reference as written: token s of the prompt is rotated by table row s (decoder_kernels.cu:440)
+    out, want, _ = run_both(gpu, 2, 4, 128, 128, 60, 20, "f32", mask=causal_mask(128), rope_row=0)
+    assert_out_close(out, want, "f32", "rope_row=0")
+
+
+def test_prefill_llama7b_shape(gpu):
+    # B=4, 32 heads, D=128, prompt of 512 tokens, fp16 caches
+    L = 640
+    out, want, _ = run_both(gpu, 4, 32, 128, L, 512, 0, "f16", mask=causal_mask(L))
+    assert_out_close(out, want, "f16", "7B prompt 512")
+
+
+def test_prefill_then_decode_steps_agree_with_oracle_sequence(gpu):
+    """Prompt of 70 tokens, then 5 decode steps on the same caches: every step against the oracle, caches
+    bit-identical at the end (the two paths write the same rows the same way)."""
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    B, H, D, L, S = 2, 4, 128, 128, 70
+    q, k, v, kc, vc, f = make(B, H, D, L, S, "f16", seed=3)
+    mask = causal_mask(L)
+    kc_ref, vc_ref = kc.copy(), vc.copy()
+    t = lambda a: torch.from_numpy(a).to(gpu)
+    op = PrefillAttention(B, H, D, L, S, torch.float16, device=gpu)
+    kc_d, vc_d, f_d, m_d = t(kc), t(vc), t(f), t(mask)
+    want = ref.prefill_attn(q, k, v, kc_ref, vc_ref, f, attn_mask=mask, acc_double=True, threads=8)
+    out = op.prefill(t(q), t(k), t(v), kc_d, vc_d, f_d, attn_mask=m_d)
+    assert_out_close(out.cpu().numpy(), want, "f16", "prompt")
+    for step in range(5):
+        qs = synth.normal((B, 1, H, D), np.float16, synth.TENSOR_Q, seed=100 + step)
+        ks = synth.normal((B, 1, H, D), np.float16, synth.TENSOR_K_NEW, seed=100 + step)
+        vs = synth.normal((B, 1, H, D), np.float16, synth.TENSOR_V_NEW, seed=100 + step)
+        w = ref.decode_attn(qs, ks, vs, kc_ref, vc_ref, f, start_pos=S + step, attn_mask=mask, acc_double=True)
+        g = op.forward(t(qs), t(ks), t(vs), kc_d, vc_d, f_d, start_pos=S + step, attn_mask=m_d)
+        assert_out_close(g.cpu().numpy(), w, "f16", f"decode step {step}")
+    assert_cache_bit_exact(kc_d.cpu().numpy(), kc_ref, "k_cache")
+    assert_cache_bit_exact(vc_d.cpu().numpy(), vc_ref, "v_cache")
+
+
+def test_prefill_equals_token_by_token_decode(gpu):
+    """With a causal mask, row s of the prompt-phase output equals the decode step at position s."""
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    B, H, D, L, S = 1, 2, 64, 64, 40
+    q, k, v, kc, vc, f = make(B, H, D, L, S, "f32", seed=9)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+    op = PrefillAttention(B, H, D, L, S, torch.float32, device=gpu)
+    f_d, m_d = t(f), t(causal_mask(L))
+    kc1, vc1 = t(kc), t(vc)
+    full = op.prefill(t(q), t(k), t(v), kc1, vc1, f_d, attn_mask=m_d).cpu().numpy()
+    kc2, vc2 = t(kc), t(vc)
+    for s in range(S):
+        o = op.forward(t(q[:, s:s + 1]), t(k[:, s:s + 1]), t(v[:, s:s + 1]), kc2, vc2, f_d, start_pos=s,
+                       attn_mask=m_d).cpu().numpy().reshape(B, H, D)
+        assert np.abs(o - full[:, :, s]).max() <= 2e-6, s
+    assert torch.equal(kc1[:, :, :S], kc2[:, :, :S]) and torch.equal(vc1[:, :, :S], vc2[:, :, :S])
+
+
+def test_prefill_int32_prologue_and_int8_epilogue(gpu):
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    B, H, D, L, S, P = 2, 8, 128, 160, 100, 0
+    rng = np.random.default_rng(8)
+    qi, ki, vi = (rng.integers(-20000, 20000, (B, S, H, D), dtype=np.int32) for _ in range(3))
+    s_in = ((rng.random((B, S)) + 0.5) * 2e-3).astype(np.float32)
+    wq, wk, wv = ((rng.random(H * D) * 3e-2 + 1e-3).astype(np.float32) for _ in range(3))
+    _, _, _, kc, vc, f = make(B, H, D, L, S, "f16")
+    mask = causal_mask(L)
+    kc_ref, vc_ref = kc.copy(), vc.copy()
+    want = ref.prefill_attn(qi, ki, vi, kc_ref, vc_ref, f, start_pos=P, attn_mask=mask, acc_double=True, threads=8,
+                            inp_scale=s_in, wq_scale=wq, wk_scale=wk, wv_scale=wv)
+    t = lambda a: torch.from_numpy(a).to(gpu)
+    op = PrefillAttention(B, H, D, L, S, torch.float16, device=gpu)
+    out = torch.empty(B, H, S, D, device=gpu)
+    q8 = torch.empty(B, S, H * D, dtype=torch.int8, device=gpu)
+    sc = torch.empty(B, S, device=gpu)
+    kc_d, vc_d = t(kc), t(vc)
+    op.prefill(t(qi), t(ki), t(vi), kc_d, vc_d, t(f), start_pos=P, out=out, attn_mask=t(mask), qkv_inp_scale=t(s_in),
+               q_weight_scale=t(wq), k_weight_scale=t(wk), v_weight_scale=t(wv), out_int8=q8, out_scale=sc)
+    torch.cuda.synchronize()
+    assert_cache_bit_exact(kc_d.cpu().numpy(), kc_ref, "k_cache")
+    assert_out_close(out.cpu().numpy(), want, "f16", "prologue")
+    q_ref, s_ref = ref.attn_quantize_transpose(out.cpu().numpy())
+    assert np.array_equal(q8.cpu().numpy(), q_ref) and np.array_equal(sc.cpu().numpy(), s_ref)
+    q_or, s_or = ref.attn_quantize_transpose(want)
+    assert np.abs(q8.cpu().numpy().astype(np.int32) - q_or.astype(np.int32)).max() <= 1
+
+
+def test_prefill_argument_errors(gpu):
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    with pytest.raises(capi.FlAttnError) as e:
+        PrefillAttention(1, 2, 256, 64, 16, torch.float16, device=gpu)
+    assert e.value.status == capi.FL_ATTN_ERR_HEAD_DIM
+    op = PrefillAttention(1, 2, 64, 64, 16, torch.float16, device=gpu)
+    z = torch.zeros(1, 16, 2, 64, dtype=torch.float16, device=gpu)
+    kc = torch.zeros(1, 2, 64, 64, dtype=torch.float16, device=gpu)
+    f = torch.zeros(64, 64, device=gpu)
+    with pytest.raises(capi.FlAttnError) as e:
+        op.prefill(z, z, z, kc, kc, f, start_pos=50)  # 50 + 16 > 64
+    assert e.value.status == capi.FL_ATTN_ERR_POSITION
+    with pytest.raises(capi.FlAttnError) as e:
+        op.prefill(z, z, z, kc, kc, f, start_pos=0, start_pos_per_seq=torch.zeros(1, dtype=torch.int32, device=gpu))
+    assert e.value.status == capi.FL_ATTN_ERR_ARGUMENT

@@ -390,3 +390,100 @@ def test_golden_fixture():
         tol_k = 2e-3 if dt == np.float16 else 4e-7
         assert np.abs(out - g[f"{name}_out"]).max() < tol_out
         assert np.abs(kc[:, :, P].astype(np.float64) - g[f"{name}_k_row"]).max() <= tol_k
+
+
+# ----------------------------------------------------------------------------- prompt phase (seq_len > 1)
+
+def make_prompt(B, H, D, L, S, dt=np.float32, seed=13):
+    q = synth.normal((B, S, H, D), dt, synth.TENSOR_Q, seed)
+    k = synth.normal((B, S, H, D), dt, synth.TENSOR_K_NEW, seed)
+    v = synth.normal((B, S, H, D), dt, synth.TENSOR_V_NEW, seed)
+    kc = synth.normal((B, H, L, D), dt, synth.TENSOR_K_CACHE, seed)
+    vc = synth.normal((B, H, L, D), dt, synth.TENSOR_V_CACHE, seed)
+    return q, k, v, kc, vc
+
+
+def causal(L, fill=-1e5):
+    return np.where(np.arange(L)[None, :] > np.arange(L)[:, None], fill, 0.0).astype(np.float32)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+def test_prefill_with_one_token_is_the_decode_step_bitwise(dt):
+    B, H, D, L, P = 2, 3, 64, 40, 17
+    q, k, v, kc, vc = make(B, H, D, L, dt)
+    f = ref.freq_cis(L, D)
+    m = (np.random.default_rng(0).standard_normal((L, L))).astype(np.float32)
+    k1, v1, k2, v2 = kc.copy(), vc.copy(), kc.copy(), vc.copy()
+    o1 = ref.decode_attn(q, k, v, k1, v1, f, start_pos=P, attn_mask=m)
+    o2 = ref.prefill_attn(q, k, v, k2, v2, f, start_pos=P, attn_mask=m)
+    assert np.array_equal(o1.ravel(), o2.ravel())
+    assert np.array_equal(k1.view(np.uint8), k2.view(np.uint8)) and np.array_equal(v1.view(np.uint8), v2.view(np.uint8))
+
+
+def test_prefill_equals_token_by_token_decode_under_a_causal_mask():
+    B, H, D, L, S, P = 2, 2, 32, 48, 20, 9
+    q, k, v, kc, vc = make_prompt(B, H, D, L, S)
+    f = ref.freq_cis(L, D)
+    m = causal(L)
+    k1, v1 = kc.copy(), vc.copy()
+    full = ref.prefill_attn(q, k, v, k1, v1, f, start_pos=P, attn_mask=m, acc_double=True)
+    k2, v2 = kc.copy(), vc.copy()
+    for s in range(S):
+        o = ref.decode_attn(np.ascontiguousarray(q[:, s:s + 1]), np.ascontiguousarray(k[:, s:s + 1]),
+                            np.ascontiguousarray(v[:, s:s + 1]), k2, v2, f, start_pos=P + s, attn_mask=m, acc_double=True)
+        assert np.abs(o.reshape(B, H, D) - full[:, :, s]).max() < 1e-6
+    assert np.array_equal(k1, k2) and np.array_equal(v1, v2)
+
+
+def test_prefill_against_torch_causal_sdpa_and_transposed_layouts():
+    torch = pytest.importorskip("torch")
+    B, H, D, L, S = 2, 3, 64, 64, 37
+    q, k, v, kc, vc = make_prompt(B, H, D, L, S)
+    f = ref.freq_cis(L, D)
+    out = ref.prefill_attn(q, k, v, kc, vc, f, start_pos=0, attn_mask=causal(L), acc_double=True)
+    assert out.shape == (B, H, S, D)
+    # appended rows: [B,S,H,D] inputs land transposed at cache[b,h,s,:]; V unchanged, K rotated by row s
+    assert np.array_equal(vc[:, :, :S], v.transpose(0, 2, 1, 3))
+    cos, sin = f[:S, 0::2][None, :, None, :], f[:S, 1::2][None, :, None, :]
+    def rot(x):
+        r = np.empty_like(x)
+        r[..., 0::2] = x[..., 0::2] * cos - x[..., 1::2] * sin
+        r[..., 1::2] = x[..., 1::2] * cos + x[..., 0::2] * sin
+        return r
+    assert np.allclose(kc[:, :, :S], rot(k).transpose(0, 2, 1, 3), atol=1e-6)
+    tq = torch.from_numpy(rot(q).transpose(0, 2, 1, 3).copy()).double()
+    tk = torch.from_numpy(kc[:, :, :S].copy()).double()
+    tv = torch.from_numpy(vc[:, :, :S].copy()).double()
+    want = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, is_causal=True).numpy()
+    assert np.abs(out - want).max() < 3e-6
+
+
+def test_prefill_chunked_prompt_attends_to_earlier_cache_rows():
+    # start_pos > 0: the keys are the cache rows [0, start_pos + S); first P rows come from the cache
+    B, H, D, L, S, P = 1, 1, 32, 32, 6, 5
+    q, k, v, kc, vc = make_prompt(B, H, D, L, S)
+    vc[:] = 0
+    for j in range(P):
+        vc[0, 0, j, j] = 1.0
+    v[:] = 0
+    for s in range(S):
+        v[0, s, 0, P + s] = 1.0
+    out = ref.prefill_attn(q, k, v, kc, vc, ref.freq_cis(L, D), start_pos=P, attn_mask=causal(L))
+    for s in range(S):
+        p = out[0, 0, s]
+        assert abs(p[:P + s + 1].sum() - 1.0) < 1e-6 and (p[:P + s + 1] > 0).all() and (p[P + s + 1:] == 0).all()
+
+
+def test_quantize_transpose_against_numpy():
+    rng = np.random.default_rng(5)
+    B, H, S, D = 2, 3, 5, 16
+    x = rng.standard_normal((B, H, S, D)).astype(np.float32)
+    qv, sc = ref.attn_quantize_transpose(x)
+    xt = x.transpose(0, 2, 1, 3).reshape(B, S, H * D)
+    absmax = np.abs(xt).max(-1)
+    assert np.array_equal(sc, (absmax / np.float32(127.0)).astype(np.float32))
+    assert np.array_equal(qv, np.clip(np.rint((xt * np.float32(127.0)) / absmax[..., None]), -128, 127).astype(np.int8))
+    # S == 1 is the decode-step quantiser
+    q1, s1 = ref.attn_quantize_transpose(x[:, :, :1])
+    q0, s0 = ref.attn_quantize(x[:, :, 0].reshape(B, H * D))
+    assert np.array_equal(q1.reshape(B, H * D), q0) and np.array_equal(s1.ravel(), s0)
