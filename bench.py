@@ -37,6 +37,95 @@ WORKLOADS = {
 }
 HEADLINE = "cfg3"
 
+# prompt-phase (seq_len > 1) shapes: a different roofline (FP32 MFMA), reported in TFLOP/s
+PREFILL_WORKLOADS = {
+    "prefill_7b_b8_s1024": dict(B=8, H=32, D=128, S=1024, P=0, L=1024, dtype="f16"),
+    "prefill_7b_b8_s1024_f32": dict(B=8, H=32, D=128, S=1024, P=0, L=1024, dtype="f32"),
+    "prefill_7b_b1_s4096": dict(B=1, H=32, D=128, S=4096, P=0, L=4096, dtype="f16"),
+    "prefill_7b_b32_s128": dict(B=32, H=32, D=128, S=128, P=0, L=256, dtype="f16"),
+}
+MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense FP32 matrix rate
+
+
+def bench_prefill(args) -> int:
+    """One step = RoPE + append + dense attention of S new tokens per sequence (prompt phase)."""
+    import numpy as np
+    import torch
+
+    from fasterllama_amd import capi, synth
+    from fasterllama_amd.decode_attn import PrefillAttention
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    capi.load()
+    dev = torch.device("cuda:0")
+    w = PREFILL_WORKLOADS[args.workload]
+    B, H, D, S, P, L = w["B"], w["H"], w["D"], w["S"], w["P"], w["L"]
+    np_dt = np.float16 if w["dtype"] == "f16" else np.float32
+    t_dt = torch.float16 if w["dtype"] == "f16" else torch.float32
+    q_h = synth.normal((B, S, H, D), np_dt, synth.TENSOR_Q, args.seed)
+    k_h = synth.normal((B, S, H, D), np_dt, synth.TENSOR_K_NEW, args.seed)
+    v_h = synth.normal((B, S, H, D), np_dt, synth.TENSOR_V_NEW, args.seed)
+    freq_h = synth.freq_cis_table(L, D)
+    mask_h = np.where(np.arange(L)[None, :] > np.arange(L)[:, None], -1e5, 0.0).astype(np.float32)  # causal
+    t = lambda a: torch.from_numpy(a).to(dev)
+    q, k, v, freq, mask = t(q_h), t(k_h), t(v_h), t(freq_h), t(mask_h)
+    kc = torch.zeros(B, H, L, D, dtype=t_dt, device=dev)
+    vc = torch.zeros_like(kc)
+    out = torch.empty(B, H, S, D, dtype=torch.float32, device=dev)
+    op = PrefillAttention(B, H, D, L, S, t_dt, device=dev)
+    io = op.make_io(q, k, v, kc, vc, freq, out, start_pos=P, attn_mask=mask)
+    stream = torch.cuda.current_stream(dev)
+
+    def run(n):
+        for _ in range(n):
+            st = op.launch_prefill(io, S, stream)
+            if st != 0:
+                raise capi.FlAttnError(st, capi.strerror(st))
+
+    steps, warm = min(args.steps, 50), min(args.warmup, 5)
+    run(warm)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    run(steps)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    flops = 4.0 * B * H * S * (P + S) * D  # every query against every key: the mask is generic, nothing is skipped
+    tflops = flops / (ms * 1e-3) / 1e12
+
+    max_err = None
+    cpu = None
+    if not args.no_cpu:
+        from oracle import ref  # checker / baseline only
+        nb = 1
+        kc_s = np.zeros((nb, H, L, D), np_dt)
+        vc_s = np.zeros_like(kc_s)
+        nthreads = max(1, min(16, os.cpu_count() or 1))
+        t1 = time.perf_counter()
+        want = ref.prefill_attn(q_h[:nb], k_h[:nb], v_h[:nb], kc_s, vc_s, freq_h, start_pos=P, attn_mask=mask_h,
+                                threads=nthreads)
+        dt_cpu = time.perf_counter() - t1
+        max_err = float(np.abs(out[:nb].cpu().numpy() - want).max())
+        cpu = {"value": round(4.0 * nb * H * S * (P + S) * D / dt_cpu / 1e12, 5), "unit": "TFLOP/s", "cores": nthreads,
+               "kind": "port", "sample": f"first {nb} of {B} sequences, scalar oracle with OpenMP over heads, {dt_cpu:.2f} s",
+               "gpu_vs_oracle_max_abs_err": max_err}
+    print(json.dumps({
+        "metric": f"prompt-phase attention TFLOP/s, {args.workload}", "value": round(tflops, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": round(ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 MFMA (f16 storage)" if w["dtype"] == "f16" else "f32 MFMA",
+        "data": "synthetic (seeded splitmix64 + Box-Muller N(0,1), seed %d)" % args.seed,
+        "config": {"workload": f"{args.workload}: B={B} H={H} D={D} S={S} start_pos={P} L={L} {w['dtype']} KV cache, "
+                               "causal additive mask (nothing skipped)", "flops_per_step": flops},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "prefill_attn_kernel (+ prefill_rope_append_kernel, same step)"},
+        "cpu_baseline": cpu}), flush=True)
+    return 0
+
 # HBM bytes per launch of the streaming kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
 # scaled by the factor the same counters read for a copy kernel of known size.  Filled in from
 # the summaries under profiles/ (None until measured for that workload).
@@ -61,7 +150,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS) + ["all"],
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS) + sorted(PREFILL_WORKLOADS) + ["all"],
                     help="'all' prints one JSON line per configuration cfg1..cfg5 (each in a child process)")
     ap.add_argument("--nsplit", type=int, default=0, help="force the context split count (0 = library's choice)")
     ap.add_argument("--seed", type=int, default=1234)
@@ -84,6 +173,9 @@ def main() -> int:
                    "--warmup", str(args.warmup), "--seed", str(args.seed)] + (["--no-cpu"] if args.no_cpu else [])
             rc |= subprocess.run(cmd).returncode
         return rc
+
+    if args.workload in PREFILL_WORKLOADS and args.gpus == 1:
+        return bench_prefill(args)
 
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path has no cross-GPU exchange); "
