@@ -43,24 +43,29 @@ namespace FasterLLaMA
     {
     }
 
-    // Workspace = the decode-step buffers of the attention segment, each 256-byte aligned:
-    //   int8 attention output | its scales | three int32 accumulator buffers | float attention output |
-    //   split partials (the larger of the two cache types' needs).
+    // Workspace = the buffers of the attention segment for up to batch_size * max_prompt_len tokens, each
+    // 256-byte aligned: int8 attention output | activation scales | three int32 accumulator buffers |
+    // output scales | scratch of the attention kernels (the largest need over both cache types and both
+    // phases; the prompt phase is left out when size_per_head is outside its supported set).
     template <OperationType OpType_, OperationType QuantizationType>
     size_t OpenDecoder<OpType_, QuantizationType>::getWorkspaceSizeBytes() const
     {
-        const size_t tokens = (size_t)batch_size_;
+        const size_t tokens = (size_t)batch_size_ * (size_t)(max_prompt_len_ > 1 ? max_prompt_len_ : 1);
         size_t n = 0;
         n += roundUp(tokens * hidden_units_ * sizeof(int8_t), 256);
         n += roundUp(tokens * sizeof(float), 256);
         n += 3 * roundUp(tokens * hidden_units_ * sizeof(int32_t), 256);
-        n += roundUp(tokens * hidden_units_ * sizeof(float), 256);
-        size_t a = 0, b = 0;
+        n += roundUp(tokens * sizeof(float), 256);
+        size_t need = 0, x = 0;
         fl_attn_desc d32 = makeDesc<float>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
         fl_attn_desc d16 = makeDesc<__half>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
-        throwOnStatus(fl_decode_attn_workspace_bytes(&d32, &a), "getWorkspaceSize");
-        throwOnStatus(fl_decode_attn_workspace_bytes(&d16, &b), "getWorkspaceSize");
-        return n + (a > b ? a : b) + 256; // slack to align a caller's base pointer
+        throwOnStatus(fl_decode_attn_workspace_bytes(&d32, &x), "getWorkspaceSize");
+        need = x;
+        throwOnStatus(fl_decode_attn_workspace_bytes(&d16, &x), "getWorkspaceSize");
+        if (x > need) need = x;
+        if (max_prompt_len_ > 1 && fl_prefill_attn_workspace_bytes(&d32, max_prompt_len_, &x) == FL_ATTN_OK && x > need)
+            need = x; // same for both cache types
+        return n + need + 256; // slack to align a caller's base pointer
     }
 
     template <OperationType OpType_, OperationType QuantizationType>
@@ -78,7 +83,7 @@ namespace FasterLLaMA
         param_ = param;
         if (!buf)
             throw std::runtime_error("[FL][ERROR] initialize: workspace is null");
-        const size_t tokens = (size_t)batch_size_;
+        const size_t tokens = (size_t)batch_size_ * (size_t)(max_prompt_len_ > 1 ? max_prompt_len_ : 1);
         char *p = reinterpret_cast<char *>(roundUp(reinterpret_cast<uintptr_t>(buf), 256));
         from_tensor_int8_buf_ = reinterpret_cast<int8_t *>(p);
         p += roundUp(tokens * hidden_units_ * sizeof(int8_t), 256);
@@ -90,7 +95,7 @@ namespace FasterLLaMA
         value_buf_ = reinterpret_cast<int32_t *>(p + 2 * acc);
         p += 3 * acc;
         qkv_buf_ = reinterpret_cast<float *>(p);
-        p += roundUp(tokens * hidden_units_ * sizeof(float), 256);
+        p += roundUp(tokens * sizeof(float), 256);
         attn_workspace_ = p;
         attn_workspace_bytes_ = getWorkspaceSizeBytes() - (size_t)(p - reinterpret_cast<char *>(roundUp(reinterpret_cast<uintptr_t>(buf), 256))) - 256;
     }
@@ -98,9 +103,9 @@ namespace FasterLLaMA
     template <OperationType OpType_, OperationType QuantizationType>
     template <typename CacheT>
     void OpenDecoder<OpType_, QuantizationType>::attentionSegment(const float *freq_cis, CacheT *key_cache, CacheT *value_cache,
-                                                                  int start_pos, const void *q, const void *k, const void *v,
-                                                                  bool int32_inputs, float *out_float, int8_t *out_int8,
-                                                                  float *out_scale)
+                                                                  int start_pos, int seq_len, const void *q, const void *k,
+                                                                  const void *v, bool int32_inputs, float *out_float,
+                                                                  int8_t *out_int8, float *out_scale)
     {
         if (!attn_workspace_)
             throw std::runtime_error("[FL][ERROR] forward: initialize() has not been called");
@@ -129,7 +134,10 @@ namespace FasterLLaMA
         }
         io.out_int8 = out_int8;
         io.out_scale = out_scale;
-        throwOnStatus(fl_decode_attn_forward(&desc, &io, param_.stream), "decode attention");
+        if (seq_len == 1)
+            throwOnStatus(fl_decode_attn_forward(&desc, &io, param_.stream), "decode attention");
+        else
+            throwOnStatus(fl_prefill_attn_forward(&desc, &io, seq_len, param_.stream), "prompt attention");
     }
 
     template <OperationType OpType_, OperationType QuantizationType>
@@ -138,24 +146,23 @@ namespace FasterLLaMA
                                                              CacheT *value_cache, DataType_ *decoder_output, int start_pos,
                                                              int seq_len)
     {
-        if (seq_len != 1)
-            throw std::runtime_error("[FL][ERROR] forward: only the decode step (seq_len == 1) is implemented; "
-                                     "the prompt phase is a dense attention outside this library");
+        if (seq_len < 1 || seq_len > (max_prompt_len_ > 1 ? max_prompt_len_ : 1))
+            throw std::runtime_error("[FL][ERROR] forward: seq_len must be between 1 and max_prompt_len");
         if (!stages_.qkv_projection || !stages_.post_attention)
             throw std::runtime_error("[FL][ERROR] forward: the Q/K/V projection and post-attention stages are external; "
                                      "install them with setExternalStages(), or call decodeAttention()");
         // RMSNorm + quantise + INT8 Q/K/V GEMMs (open_decoder.cu:92-136) -> int32 accumulators
         stages_.qkv_projection(stages_.user, from_tensor, query_buf_, key_buf_, value_buf_, from_tensor_scale_buf_, batch_size_,
-                               param_.stream);
+                               seq_len, param_.stream);
         // dequantise + RoPE + cache append + attention + per-token INT8 quantisation (open_decoder.cu:138-246).
         // The reference reuses from_tensor_scale_buf_ for the output scale; here the quantised output gets
-        // its own slot (the head of the unused float-output buffer) so the activation scale stays readable.
+        // its own slot so the activation scale stays readable.
         float *attn_scale = qkv_buf_;
-        attentionSegment<CacheT>(freq_cis, key_cache, value_cache, start_pos, query_buf_, key_buf_, value_buf_, true, nullptr,
-                                 from_tensor_int8_buf_, attn_scale);
+        attentionSegment<CacheT>(freq_cis, key_cache, value_cache, start_pos, seq_len, query_buf_, key_buf_, value_buf_, true,
+                                 nullptr, from_tensor_int8_buf_, attn_scale);
         // output projection, residual, FFN (open_decoder.cu:256-346)
         stages_.post_attention(stages_.user, from_tensor_int8_buf_, attn_scale, from_tensor, decoder_output, batch_size_,
-                               param_.stream);
+                               seq_len, param_.stream);
     }
 
     template <OperationType OpType_, OperationType QuantizationType>
@@ -179,7 +186,7 @@ namespace FasterLLaMA
                                                                  float *key_cache_, float *value_cache_, float *attn_out,
                                                                  int start_pos)
     {
-        attentionSegment<float>(freq_cis, key_cache_, value_cache_, start_pos, q, k, v, false, attn_out, nullptr, nullptr);
+        attentionSegment<float>(freq_cis, key_cache_, value_cache_, start_pos, 1, q, k, v, false, attn_out, nullptr, nullptr);
     }
 
     template <OperationType OpType_, OperationType QuantizationType>
@@ -187,7 +194,7 @@ namespace FasterLLaMA
                                                                  const float *freq_cis, __half *key_cache_, __half *value_cache_,
                                                                  float *attn_out, int start_pos)
     {
-        attentionSegment<__half>(freq_cis, key_cache_, value_cache_, start_pos, q, k, v, false, attn_out, nullptr, nullptr);
+        attentionSegment<__half>(freq_cis, key_cache_, value_cache_, start_pos, 1, q, k, v, false, attn_out, nullptr, nullptr);
     }
 
     template <OperationType OpType_, OperationType QuantizationType>

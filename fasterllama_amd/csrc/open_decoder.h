@@ -4,12 +4,12 @@
 //   fasterLlama/open_decoder.h:8-23   DecoderInitParam
 //   fasterLlama/open_decoder.h:26-79  OpenDecoder {ctor, initialize, getWorkspaceSize, forward}
 //   fasterLlama/cuda/common.h:9-47    OperationType and the weight structs
-// so a caller written against the reference compiles against this header.  Only the decode-step
-// attention segment of forward() (open_decoder.cu:138-246, seq_len == 1) is implemented here — by
-// one call into the C ABI of libfl_decode_attn.  The stages before it (RMSNorm + INT8 Q/K/V
-// projections, open_decoder.cu:92-136) and after it (output projection and FFN,
-// open_decoder.cu:256-346) are dense INT8 GEMM work outside this library; forward() reaches them
-// through the two callbacks of DecoderExternalStages.
+// so a caller written against the reference compiles against this header.  Only the attention
+// segment of forward() (open_decoder.cu:138-246) is implemented here — by one call into the C ABI of
+// libfl_decode_attn: the decode step (seq_len == 1) and the prompt phase (seq_len > 1).  The stages
+// before it (RMSNorm + INT8 Q/K/V projections, open_decoder.cu:92-136) and after it (output
+// projection and FFN, open_decoder.cu:256-346) are dense INT8 GEMM work outside this library;
+// forward() reaches them through the two callbacks of DecoderExternalStages.
 //
 // Differences a caller sees, all forced by the platform or by defects of the reference:
 //   - DecoderInitParam::stream is a hipStream_t; cublas_handle is an opaque pointer that the
@@ -98,14 +98,14 @@ namespace FasterLLaMA
     struct DecoderExternalStages
     {
         void *user = nullptr;
-        // from_tensor [B, hidden] -> int32 accumulators of the INT8 Q/K/V projections, each
-        // [B, head_num * size_per_head], and the per-token activation scale [B].
+        // from_tensor [B*seq_len, hidden] -> int32 accumulators of the INT8 Q/K/V projections, each
+        // [B*seq_len, head_num * size_per_head], and the per-token activation scale [B*seq_len].
         void (*qkv_projection)(void *user, const T *from_tensor, int32_t *query_buf, int32_t *key_buf,
-                               int32_t *value_buf, float *from_tensor_scale_buf, int batch_size,
+                               int32_t *value_buf, float *from_tensor_scale_buf, int batch_size, int seq_len,
                                hipStream_t stream) = nullptr;
-        // attention output, INT8 [B, hidden] with its per-token scale [B] -> decoder_output
+        // attention output, INT8 [B*seq_len, hidden] with its per-token scale [B*seq_len] -> decoder_output
         void (*post_attention)(void *user, const int8_t *attn_int8, const float *attn_scale,
-                               const T *from_tensor, T *decoder_output, int batch_size,
+                               const T *from_tensor, T *decoder_output, int batch_size, int seq_len,
                                hipStream_t stream) = nullptr;
     };
 
@@ -133,17 +133,18 @@ namespace FasterLLaMA
         int nsplit_ = 0;
 
         // carved from the caller's workspace by initialize(); names follow open_decoder.h:53-64
-        int8_t *from_tensor_int8_buf_ = nullptr;  // [B, hidden] attention output, quantised
-        float *from_tensor_scale_buf_ = nullptr;  // [B]
-        int32_t *query_buf_ = nullptr;            // [B, hidden]
-        int32_t *key_buf_ = nullptr;              // [B, hidden]
-        int32_t *value_buf_ = nullptr;            // [B, hidden]
-        float *qkv_buf_ = nullptr;                // [B, hidden] attention output, float
-        char *attn_workspace_ = nullptr;          // split partials of the attention kernels
+        // (tokens = batch_size * max_prompt_len)
+        int8_t *from_tensor_int8_buf_ = nullptr;  // [tokens, hidden] attention output, quantised
+        float *from_tensor_scale_buf_ = nullptr;  // [tokens]
+        int32_t *query_buf_ = nullptr;            // [tokens, hidden]
+        int32_t *key_buf_ = nullptr;              // [tokens, hidden]
+        int32_t *value_buf_ = nullptr;            // [tokens, hidden]
+        float *qkv_buf_ = nullptr;                // [tokens] output scales of the quantised attention output
+        char *attn_workspace_ = nullptr;          // scratch of the attention kernels
         size_t attn_workspace_bytes_ = 0;
 
         template <typename CacheT>
-        void attentionSegment(const float *freq_cis, CacheT *key_cache, CacheT *value_cache, int start_pos,
+        void attentionSegment(const float *freq_cis, CacheT *key_cache, CacheT *value_cache, int start_pos, int seq_len,
                               const void *q, const void *k, const void *v, bool int32_inputs, float *out_float,
                               int8_t *out_int8, float *out_scale);
         template <typename CacheT>
@@ -161,8 +162,8 @@ namespace FasterLLaMA
 
         /**
          * key_cache_, value_cache_: [batch_size, head_num, total_len_, size_per_head]
-         * freq_cis: [rows >= start_pos + 1, size_per_head]
-         * Only seq_len == 1 (one new token per sequence) is implemented; other values throw.
+         * freq_cis: [rows >= start_pos + seq_len, size_per_head]
+         * seq_len == 1: decode step; 1 < seq_len <= max_prompt_len: prompt phase (size_per_head 32/64/128).
          */
         void forward(const DataType_ *from_tensor, const float *freq_cis, float *key_cache_, float *value_cache_,
                      DataType_ *decoder_output, const int start_pos, const int seq_len);

@@ -24,6 +24,11 @@ int fl_ref_decode_attn_i32(int dtype, int B, int H, int D, int L, const int32_t 
                            const float *attn_mask, int64_t mask_ld, int start_pos, const int32_t *start_pos_per_seq,
                            float scale, float *out, int acc_double, int threads);
 int fl_ref_attn_quantize(int B, int HD, const float *attn, int8_t *out_q, float *out_scale);
+int fl_ref_prefill_attn(int dtype, int B, int H, int D, int L, int S, const void *q, const void *k_new, const void *v_new,
+                        const float *inp_scale, const float *wq_scale, const float *wk_scale, const float *wv_scale,
+                        void *k_cache, void *v_cache, const float *freq_cis, int rope_row, const float *attn_mask,
+                        int64_t mask_ld, int start_pos, float scale, float *out, int acc_double, int threads);
+int fl_ref_attn_quantize_transpose(int B, int H, int S, int D, const float *attn, int8_t *out_q, float *out_scale);
 int fl_ref_freq_cis(float *table, int rows, int D, double base);
 uint16_t fl_ref_float_to_half(float f);
 }
@@ -73,9 +78,10 @@ struct HookCtx {
 };
 
 template <typename T>
-static void qkvHook(void *user, const T *, int32_t *qb, int32_t *kb, int32_t *vb, float *sb, int B, hipStream_t s)
+static void qkvHook(void *user, const T *, int32_t *qb, int32_t *kb, int32_t *vb, float *sb, int B, int S, hipStream_t s)
 {
     HookCtx *c = static_cast<HookCtx *>(user);
+    B *= S; // tokens
     const size_t bytes = (size_t)B * c->hidden * sizeof(int32_t);
     HIP_OK(hipMemcpyAsync(qb, c->q, bytes, hipMemcpyDeviceToDevice, s));
     HIP_OK(hipMemcpyAsync(kb, c->k, bytes, hipMemcpyDeviceToDevice, s));
@@ -85,9 +91,10 @@ static void qkvHook(void *user, const T *, int32_t *qb, int32_t *kb, int32_t *vb
 }
 
 template <typename T>
-static void postHook(void *user, const int8_t *a8, const float *as, const T *, T *, int B, hipStream_t s)
+static void postHook(void *user, const int8_t *a8, const float *as, const T *, T *, int B, int S, hipStream_t s)
 {
     HookCtx *c = static_cast<HookCtx *>(user);
+    B *= S; // tokens
     HIP_OK(hipMemcpyAsync(c->seen_int8, a8, (size_t)B * c->hidden, hipMemcpyDeviceToDevice, s));
     HIP_OK(hipMemcpyAsync(c->seen_scale, as, (size_t)B * sizeof(float), hipMemcpyDeviceToDevice, s));
     c->calls_post++;
@@ -181,13 +188,13 @@ template <OperationType Op, typename CacheT> static void runAll(const char *tag)
     DevBuf<int8_t> d_seen8((size_t)B * HD);
     DevBuf<float> d_seens(B);
     HookCtx ctx{d_qi.p, d_ki.p, d_vi.p, d_sin.p, d_seen8.p, d_seens.p, (size_t)HD};
+    DecoderExternalStages<DataT> stages_keep;
     {
         d_kc.up(kc.data()); d_vc.up(vc.data());
-        DecoderExternalStages<DataT> stages;
-        stages.user = &ctx;
-        stages.qkv_projection = qkvHook<DataT>;
-        stages.post_attention = postHook<DataT>;
-        dec.setExternalStages(stages);
+        stages_keep.user = &ctx;
+        stages_keep.qkv_projection = qkvHook<DataT>;
+        stages_keep.post_attention = postHook<DataT>;
+        dec.setExternalStages(stages_keep);
         DevBuf<DataT> d_from((size_t)B * HD), d_dec_out((size_t)B * HD);
         dec.forward(d_from.p, d_freq.p, d_kc.p, d_vc.p, d_dec_out.p, P, 1);
         HIP_OK(hipStreamSynchronize(stream));
@@ -229,11 +236,56 @@ template <OperationType Op, typename CacheT> static void runAll(const char *tag)
         report(name, same);
     }
 
+    // ---- 3b. prompt phase through forward(): seq_len = 24 tokens at start_pos 0 (the reference's prefill call)
+    {
+        const int S = 24;
+        std::vector<int32_t> pq((size_t)B * S * HD), pk(pq.size()), pv(pq.size());
+        for (auto &x : pq) x = (int32_t)(frand() * 20000.f);
+        for (auto &x : pk) x = (int32_t)(frand() * 20000.f);
+        for (auto &x : pv) x = (int32_t)(frand() * 20000.f);
+        std::vector<float> ps((size_t)B * S);
+        for (auto &x : ps) x = 0.002f + 0.001f * (frand() + 1.0f);
+        DevBuf<int32_t> d_pq(pq.size()), d_pk(pk.size()), d_pv(pv.size());
+        DevBuf<float> d_ps(ps.size()), d_seens2((size_t)B * S);
+        DevBuf<int8_t> d_seen82((size_t)B * S * HD);
+        d_pq.up(pq.data()); d_pk.up(pk.data()); d_pv.up(pv.data()); d_ps.up(ps.data());
+        d_kc.up(kc.data()); d_vc.up(vc.data());
+        HookCtx pctx{d_pq.p, d_pk.p, d_pv.p, d_ps.p, d_seen82.p, d_seens2.p, (size_t)HD};
+        DecoderExternalStages<DataT> st2;
+        st2.user = &pctx;
+        st2.qkv_projection = qkvHook<DataT>;
+        st2.post_attention = postHook<DataT>;
+        dec.setExternalStages(st2);
+        DevBuf<DataT> d_from((size_t)B * S * HD), d_dec_out((size_t)B * S * HD);
+        dec.forward(d_from.p, d_freq.p, d_kc.p, d_vc.p, d_dec_out.p, 0, S);
+        HIP_OK(hipStreamSynchronize(stream));
+
+        std::vector<CacheT> kc_ref(kc), vc_ref(vc), kc_got(kc.size());
+        std::vector<float> want((size_t)B * H * S * D), want_s((size_t)B * S), got_s(want_s.size());
+        std::vector<int8_t> want8((size_t)B * S * HD), got8(want8.size());
+        fl_ref_prefill_attn(code, B, H, D, L, S, pq.data(), pk.data(), pv.data(), ps.data(), wq.data(), wk.data(), wv.data(),
+                            kc_ref.data(), vc_ref.data(), freq.data(), -1, mask.data(), L, 0, 1.0f / std::sqrt((float)D),
+                            want.data(), 1, 4);
+        fl_ref_attn_quantize_transpose(B, H, S, D, want.data(), want8.data(), want_s.data());
+        d_seen82.down(got8.data()); d_seens2.down(got_s.data()); d_kc.down(kc_got.data());
+        int worst8 = 0;
+        for (size_t i = 0; i < want8.size(); ++i) worst8 = std::max(worst8, std::abs((int)got8[i] - (int)want8[i]));
+        double worst_s = 0;
+        for (size_t i = 0; i < want_s.size(); ++i) worst_s = std::fmax(worst_s, std::fabs(got_s[i] - want_s[i]) / want_s[i]);
+        std::snprintf(name, sizeof name, "%s prompt forward int8 within one step", tag);
+        report(name, worst8 <= 1 && pctx.calls_pre == 1 && pctx.calls_post == 1, worst8);
+        std::snprintf(name, sizeof name, "%s prompt forward output scale", tag);
+        report(name, worst_s <= 1e-5, worst_s);
+        std::snprintf(name, sizeof name, "%s prompt forward k_cache bit-exact", tag);
+        report(name, !std::memcmp(kc_got.data(), kc_ref.data(), kc.size() * sizeof(CacheT)));
+        dec.setExternalStages(stages_keep);
+    }
+
     // ---- 4. error behaviour: std::runtime_error, never exit()
     {
         DevBuf<DataT> d_from((size_t)B * HD), d_dec_out((size_t)B * HD);
         int caught = 0;
-        try { dec.forward(d_from.p, d_freq.p, d_kc.p, d_vc.p, d_dec_out.p, 0, 2); } catch (std::runtime_error &) { caught++; }
+        try { dec.forward(d_from.p, d_freq.p, d_kc.p, d_vc.p, d_dec_out.p, 0, prompt + 1); } catch (std::runtime_error &) { caught++; }
         try { dec.forward(d_from.p, d_freq.p, d_kc.p, d_vc.p, d_dec_out.p, L, 1); } catch (std::runtime_error &) { caught++; }
         try { dec.decodeAttention(d_q.p, d_k.p, d_v.p, (const float *)nullptr, d_kc.p, d_vc.p, d_out.p, P); } catch (std::runtime_error &) { caught++; }
         try {
