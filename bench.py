@@ -34,6 +34,9 @@ WORKLOADS = {
     # exploration shapes (not among the five headline configurations)
     "x13b_uniform": dict(B=32, H=40, D=128, ctx=4096, L=4096, dtype="f16", copies=1),
     "x7b_halffull": dict(B=64, H=32, D=128, ctx=2048, L=4096, dtype="f16", copies=1),
+    "x7b_f32": dict(B=64, H=32, D=128, ctx=2048, L=2048, dtype="f32", copies=1),  # the reference's cache type
+    "xd64": dict(B=64, H=64, D=64, ctx=2048, L=2048, dtype="f16", copies=1),
+    "xd256": dict(B=64, H=16, D=256, ctx=2048, L=2048, dtype="f16", copies=1),
 }
 HEADLINE = "cfg3"
 
@@ -131,7 +134,7 @@ def bench_prefill(args) -> int:
 # the summaries under profiles/ (None until measured for that workload).
 MEASURED_TRAFFIC_BYTES = {
     # profiles/decode_attn_split_kernel_f16_b64_h32_d128_ctx2048.md
-    "cfg3": 2150680000,
+    "cfg3": 2150757750,
 }
 
 
