@@ -35,6 +35,12 @@ WORKLOADS = {
     "x13b_uniform": dict(B=32, H=40, D=128, ctx=4096, L=4096, dtype="f16", copies=1),
     "x7b_halffull": dict(B=64, H=32, D=128, ctx=2048, L=4096, dtype="f16", copies=1),
     "x7b_f32": dict(B=64, H=32, D=128, ctx=2048, L=2048, dtype="f32", copies=1),  # the reference's cache type
+    "xb80": dict(B=80, H=32, D=128, ctx=2048, L=2048, dtype="f16", copies=1),
+    "xb48": dict(B=48, H=32, D=128, ctx=2048, L=2048, dtype="f16", copies=1),
+    "xb100": dict(B=100, H=32, D=128, ctx=1024, L=1024, dtype="f16", copies=1),
+    "xb32": dict(B=32, H=32, D=128, ctx=2048, L=2048, dtype="f16", copies=1),
+    "xb16": dict(B=16, H=32, D=128, ctx=2048, L=2048, dtype="f16", copies=1),
+    "xb4": dict(B=4, H=32, D=128, ctx=2048, L=2048, dtype="f16", copies=4),
     "xd64": dict(B=64, H=64, D=64, ctx=2048, L=2048, dtype="f16", copies=1),
     "xd256": dict(B=64, H=16, D=256, ctx=2048, L=2048, dtype="f16", copies=1),
 }

@@ -88,12 +88,14 @@ int unroll_for(const fl_attn_desc *d)
 }
 
 // ---- launch planning ---------------------------------------------------------------------------
-// slots = workgroups the device holds at once (8 four-wave workgroups per CU at 64 VGPRs).
-// Uniform batches: when B*H fills the slots, one split per (b,h) (no partials, no combine pass) unless
-// a fractional last round of workgroups would idle much of the chip, in which case 2-4 splits smooth
-// it; when B*H is smaller, floor(slots / (B*H)) splits fill the device in a single round.
-// Ragged batches (per-sequence positions on the device): work per (b,h) varies, so splits are also
-// capped at ~256 KB of K+V per workgroup, which measured best on 13B-shaped ragged batches.
+// A streaming workgroup alone pulls about 23 GB/s (one 64-row tile of 32 KB per ~1.4 us with eight
+// 16-byte loads per lane in flight), so about one workgroup per compute unit already saturates HBM
+// (measured: 256 workgroups reach 5.9 TB/s, 512 reach 6.9 TB/s).  Splitting the context buys nothing
+// beyond that and costs the partial traffic plus a combine launch (~3.5 us), so:
+//   uniform batches: nsplit = ceil(CUs / (B*H)), never finer than one tile per split, and contexts
+//   of at most four tiles stay whole;
+//   ragged batches (per-sequence positions on the device): work per (b,h) varies, so splits are
+//   also capped at ~256 KB of K+V per workgroup, which measured best on 13B-shaped ragged batches.
 constexpr size_t kRaggedChunkBytes = 256 * 1024;
 
 int row_bytes(const fl_attn_desc *d) { return d->size_per_head * (d->dtype == FL_ATTN_F16 ? 2 : 4); }
@@ -107,20 +109,8 @@ int min_chunk_rows(const fl_attn_desc *d)
 int uniform_splits(const fl_attn_desc *d, int ctx)
 {
     const int64_t bh = (int64_t)d->batch_size * d->head_num;
-    const int64_t slots = (int64_t)device_cus() * 8;
-    int64_t n;
-    if (bh <= slots) {
-        n = slots / bh;
-    } else {
-        // estimated cost of n splits: idle fraction of the last round, plus ~2% for the combine pass
-        double best = 1e30;
-        n = 1;
-        for (int c = 1; c <= 4; ++c) {
-            const double rounds = (double)(bh * c) / (double)slots;
-            const double cost = std::ceil(rounds) / rounds * (c > 1 ? 1.02 : 1.0);
-            if (cost < best - 1e-9) { best = cost; n = c; }
-        }
-    }
+    const int64_t cus = device_cus();
+    int64_t n = (cus + bh - 1) / bh;
     const int64_t most = ((int64_t)ctx + min_chunk_rows(d) - 1) / min_chunk_rows(d);
     if (n > most) n = most;
     // a combine launch costs about as much as streaming three more tiles in one workgroup

@@ -149,18 +149,20 @@ def test_plans_cover_the_context_and_respect_forced_splits():
 
 
 def test_plan_heuristics_at_the_benchmark_shapes():
-    """Without a GPU the library assumes 256 compute units (2048 resident workgroups)."""
+    """Without a GPU the library assumes 256 compute units; about one streaming workgroup per
+    compute unit saturates HBM, so contexts are split only when B*H is smaller than that."""
     lib = capi.load()
     plan = capi.AttnPlan()
-    # headline: B*H = 2048 fills the device -> single pass, no partials
+    # headline: B*H = 2048 -> single pass, no partials
     d = desc(B=64, H=32, D=128, L=2048)
     assert lib.fl_decode_attn_plan(C.byref(d), 2048, 0, C.byref(plan)) == 0 and (plan.nsplit, plan.two_pass) == (1, 0)
-    # B=8: 256 (b,h) pairs -> 8 splits of 128 rows fill the device in one round
+    # B=8: 256 (b,h) pairs already fill the device -> no split either
     d = desc(B=8, H=32, D=128, L=1024)
-    assert lib.fl_decode_attn_plan(C.byref(d), 1024, 0, C.byref(plan)) == 0 and (plan.nsplit, plan.chunk_rows) == (8, 128)
-    # B=1, ctx 4096: 64 splits of 64 rows
+    assert lib.fl_decode_attn_plan(C.byref(d), 1024, 0, C.byref(plan)) == 0 and (plan.nsplit, plan.chunk_rows) == (1, 1024)
+    # B=1, ctx 4096: 32 pairs -> 8 splits of 512 rows
     d = desc(B=1, H=32, D=128, L=4096)
-    assert lib.fl_decode_attn_plan(C.byref(d), 4096, 0, C.byref(plan)) == 0 and (plan.nsplit, plan.chunk_rows) == (64, 64)
+    assert lib.fl_decode_attn_plan(C.byref(d), 4096, 0, C.byref(plan)) == 0 and (plan.nsplit, plan.chunk_rows) == (8, 512)
+    assert lib.fl_decode_attn_plan(C.byref(d), 200, 0, C.byref(plan)) == 0 and plan.nsplit == 1  # short contexts stay whole
     # ragged 13B batch: ~256 KB of K+V per workgroup -> 512-row chunks
     d = desc(B=32, H=40, D=128, L=4096)
     assert lib.fl_decode_attn_plan(C.byref(d), 4096, 1, C.byref(plan)) == 0 and (plan.nsplit, plan.chunk_rows) == (8, 512)
