@@ -53,7 +53,8 @@ PREFILL_WORKLOADS = {
     "prefill_7b_b1_s4096": dict(B=1, H=32, D=128, S=4096, P=0, L=4096, dtype="f16"),
     "prefill_7b_b32_s128": dict(B=32, H=32, D=128, S=128, P=0, L=256, dtype="f16"),
 }
-MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense FP32 matrix rate
+MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X published dense FP32 matrix rate (FP32 caches)
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 matrix rate (fp16 caches)
 
 
 def bench_prefill(args) -> int:
@@ -84,7 +85,7 @@ def bench_prefill(args) -> int:
     vc = torch.zeros_like(kc)
     out = torch.empty(B, H, S, D, dtype=torch.float32, device=dev)
     op = PrefillAttention(B, H, D, L, S, t_dt, device=dev)
-    io = op.make_io(q, k, v, kc, vc, freq, out, start_pos=P, attn_mask=mask)
+    io = op.make_io(q, k, v, kc, vc, freq, out, start_pos=P, attn_mask=mask if args.prefill_mask == "causal" else None)
     stream = torch.cuda.current_stream(dev)
 
     def run(n):
@@ -104,6 +105,7 @@ def bench_prefill(args) -> int:
     ms = e0.elapsed_time(e1) / steps
     flops = 4.0 * B * H * S * (P + S) * D  # every query against every key: the mask is generic, nothing is skipped
     tflops = flops / (ms * 1e-3) / 1e12
+    peak = MFMA_FP16_PEAK_TFLOPS if w["dtype"] == "f16" else MFMA_FP32_PEAK_TFLOPS
 
     max_err = None
     cpu = None
@@ -114,8 +116,8 @@ def bench_prefill(args) -> int:
         vc_s = np.zeros_like(kc_s)
         nthreads = max(1, min(16, os.cpu_count() or 1))
         t1 = time.perf_counter()
-        want = ref.prefill_attn(q_h[:nb], k_h[:nb], v_h[:nb], kc_s, vc_s, freq_h, start_pos=P, attn_mask=mask_h,
-                                threads=nthreads)
+        want = ref.prefill_attn(q_h[:nb], k_h[:nb], v_h[:nb], kc_s, vc_s, freq_h, start_pos=P,
+                                attn_mask=mask_h if args.prefill_mask == "causal" else None, threads=nthreads)
         dt_cpu = time.perf_counter() - t1
         max_err = float(np.abs(out[:nb].cpu().numpy() - want).max())
         cpu = {"value": round(4.0 * nb * H * S * (P + S) * D / dt_cpu / 1e12, 5), "unit": "TFLOP/s", "cores": nthreads,
@@ -125,12 +127,13 @@ def bench_prefill(args) -> int:
         "metric": f"prompt-phase attention TFLOP/s, {args.workload}", "value": round(tflops, 2), "unit": "TFLOP/s",
         "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": round(ms, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32 MFMA (f16 storage)" if w["dtype"] == "f16" else "f32 MFMA",
+        "dtype": "f16 MFMA, f32 accumulate (f16 storage)" if w["dtype"] == "f16" else "f32 MFMA",
         "data": "synthetic (seeded splitmix64 + Box-Muller N(0,1), seed %d)" % args.seed,
         "config": {"workload": f"{args.workload}: B={B} H={H} D={D} S={S} start_pos={P} L={L} {w['dtype']} KV cache, "
-                               "causal additive mask (nothing skipped)", "flops_per_step": flops},
-        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": None,
+                               + ("causal additive mask (nothing skipped)" if args.prefill_mask == "causal" else "no mask"),
+                   "flops_per_step": flops},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(tflops / peak, 4), "traffic": None,
                      "kernel": "prefill_attn_kernel (+ prefill_rope_append_kernel, same step)"},
         "cpu_baseline": cpu}), flush=True)
     return 0
@@ -168,6 +171,8 @@ def main() -> int:
                     help="only run a plain 1 GiB -> 1 GiB elementwise copy kernel a few times (for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings), then exit")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
+    ap.add_argument("--prefill-mask", default="causal", choices=["causal", "none"],
+                    help="prompt-phase workloads: additive causal mask (as the reference passes) or no mask")
     ap.add_argument("--segment", default="attention", choices=["attention", "int32-int8"],
                     help="attention: q/k/v in the cache dtype -> float output (the headline metric). "
                          "int32-int8: the whole reference segment, int32 GEMM accumulators + scales in, "

@@ -262,10 +262,17 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
     if (e != hipSuccess) return e;
     const unsigned qblocks = (unsigned)((p.S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock);
     const dim3 grid(qblocks * (unsigned)(p.B * p.H)); // (b,h) fastest: the query blocks of one head share an XCD's L2
-    if (p.attn_mask)
-        hipLaunchKernelGGL((flattn::prefill_attn_kernel<T, D, true>), grid, dim3(256), 0, stream, p);
-    else
-        hipLaunchKernelGGL((flattn::prefill_attn_kernel<T, D, false>), grid, dim3(256), 0, stream, p);
+    if constexpr (std::is_same<T, _Float16>::value) {
+        if (p.attn_mask)
+            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, true>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, false>), grid, dim3(256), 0, stream, p);
+    } else {
+        if (p.attn_mask)
+            hipLaunchKernelGGL((flattn::prefill_attn_kernel<T, D, true>), grid, dim3(256), 0, stream, p);
+        else
+            hipLaunchKernelGGL((flattn::prefill_attn_kernel<T, D, false>), grid, dim3(256), 0, stream, p);
+    }
     return hipGetLastError();
 }
 

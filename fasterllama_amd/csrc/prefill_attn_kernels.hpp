@@ -5,8 +5,10 @@
 //   block softmax with mask row start_pos + q  (decoder_kernels.cu:800-835)
 //   out = P V       (cublasGemmStridedBatchedEx, open_decoder.cu:218-227)
 // Unlike the decode step this is a dense contraction (S x ctx x D per head), so it runs on the
-// matrix cores: FP32 MFMA (v_mfma_f32_32x32x2_f32) with FP32 operands, which keeps the 1e-5
-// parity bar of the FP32 path; fp16 caches are widened to FP32 when a tile is staged in LDS.
+// matrix cores.  FP32 caches: FP32 MFMA (v_mfma_f32_32x32x2_f32) with FP32 operands, which keeps the
+// 1e-5 parity bar of the FP32 path.  fp16 caches: fp16 MFMA (v_mfma_f32_32x32x16_f16) with FP32
+// accumulation (prefill_attn_f16_kernel); the FP32-MFMA kernel also accepts fp16 caches, widening
+// them when a tile is staged in LDS.
 //
 // Two kernels:
 //   prefill_rope_append_kernel  elementwise: RoPE(q) -> workspace [B,H,S,D] fp32, RoPE(k), v ->
@@ -101,6 +103,31 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kPrefillQueriesPerBlock = 128; // 4 waves x 32 queries
 constexpr int kPrefillKeysPerStep = 32;
+constexpr int kMaskTileLd = kPrefillKeysPerStep + 4; // padded: 128-bit reads of 8 consecutive rows hit 32 banks
+
+// Stages the additive-mask tile of a workgroup (128 queries x 32 keys, rows start_pos + q of the
+// caller's [*, mask_ld] matrix) in LDS with coalesced loads: 256 cache-line reads per tile, where
+// per-lane gathers (each lane a different mask row) cost 4096 and made the texture path the bottleneck
+// of the fp16 kernel.  Entries outside the prompt or the context are 0 (their scores are forced to
+// -inf or never used).  `mul` pre-scales the mask for the base-2 softmax.
+__device__ __forceinline__ void stage_mask_tile(const PrefillParams &p, float (*sM)[kMaskTileLd], int qb, int k0, int ctx,
+                                                int tid, float mul)
+{
+    // thread -> (row r0 + 8j, column c): 32 consecutive lanes read one 128-byte row segment
+    const int c = tid & 31, r0 = tid >> 5;
+    const int q0 = qb * kPrefillQueriesPerBlock + r0;
+    const bool key_ok = k0 + c < ctx;
+    const float *src = p.attn_mask + (size_t)(p.start_pos + q0) * p.mask_ld + k0 + c;
+    const size_t step = (size_t)8 * p.mask_ld;
+    float x[kPrefillQueriesPerBlock / 8];
+#pragma unroll
+    for (int j = 0; j < kPrefillQueriesPerBlock / 8; ++j) { // all 16 loads in flight together
+        x[j] = 0.f;
+        if (key_ok && q0 + 8 * j < p.S) x[j] = src[j * step];
+    }
+#pragma unroll
+    for (int j = 0; j < kPrefillQueriesPerBlock / 8; ++j) sM[r0 + 8 * j][c] = x[j] * mul;
+}
 
 // MFMA operand layouts used below (v_mfma_f32_32x32x2_f32, D += A(32x2) * B(2x32)):
 //   A: lane holds A[row = lane % 32][k = lane / 32];  B: lane holds B[k = lane / 32][col = lane % 32];
@@ -176,6 +203,9 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
                 *reinterpret_cast<float4 *>(&sV[r][cc * VEC + i]) = make_float4(vf[i], vf[i + 1], vf[i + 2], vf[i + 3]);
             }
         }
+        // mask values of this lane's query, gathered straight from global memory: the FP32-MFMA kernel
+        // is matrix-core bound with every register in use, so the gather hides behind the products
+        // (staging the tile in LDS, as the fp16 kernel does, costs occupancy here: 1.53 -> 2.09 ms)
         float mk[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -242,6 +272,167 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
             for (int g4 = 0; g4 < 4; ++g4) {
                 float4 r;
                 r.x = ot[dt][4 * g4 + 0] / l; // p = e / sum (decoder_kernels.cu:833)
+                r.y = ot[dt][4 * g4 + 1] / l;
+                r.z = ot[dt][4 * g4 + 2] / l;
+                r.w = ot[dt][4 * g4 + 3] / l;
+                *reinterpret_cast<float4 *>(dst + 32 * dt + 8 * g4 + 4 * hf) = r;
+            }
+    }
+}
+
+// ---------------------------------------------------------------- fp16 caches: fp16 MFMA
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+
+// Same algorithm as prefill_attn_kernel for fp16 caches, on v_mfma_f32_32x32x16_f16: K and V tiles
+// stay fp16 in LDS (V transposed, so a lane fetches the eight keys of one MFMA as two 64-bit reads),
+// rotated queries and probabilities are rounded to fp16 as MFMA operands, every accumulation is
+// FP32 (scores, softmax statistics, output).  The rounding of q and p costs ~1e-4 absolute on the
+// output, inside the 2e-3 bar of the fp16 path.  The softmax runs in base 2 like the fp16 decode
+// kernels.  Contraction slots: a lane-half hf supplies eight consecutive slots of each MFMA; for the
+// first product they are d = 16c + 8hf + r, for the second the keys this lane holds after the first:
+// 16u + 4hf + r (r < 4) and 16u + 8 + 4hf + (r - 4).
+// three waves per SIMD (<= 170 registers, accumulators in VGPRs): 0.56 -> 0.48 ms at B=8, S=1024
+#ifndef FLATTN_PREFILL_F16_WAVES
+#define FLATTN_PREFILL_F16_WAVES 3
+#endif
+template <int D, bool HAS_MASK>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(FLATTN_PREFILL_F16_WAVES, 8)))
+void prefill_attn_f16_kernel(const PrefillParams p)
+{
+    constexpr int BN = kPrefillKeysPerStep; // 32
+    constexpr int LDK = D + 8;              // halfs; rows start 4 banks apart
+    constexpr int LDV = BN + 4;             // halfs; 18-dword rows: 16 lanes x 64-bit reads hit 32 distinct banks
+    constexpr int NC = D / 16;
+    constexpr int NDT = D / 32;
+    constexpr int CPR = D / 8; // 16-byte chunks per cache row
+    static_assert(D % 32 == 0, "head size must be a multiple of 32");
+
+    __shared__ __attribute__((aligned(16))) _Float16 sK[BN][LDK];
+    __shared__ __attribute__((aligned(16))) _Float16 sVt[D][LDV];
+    __shared__ float sM[HAS_MASK ? kPrefillQueriesPerBlock : 1][kMaskTileLd];
+
+    const int BH = p.B * p.H;
+    const int qb = blockIdx.x / BH, bh = blockIdx.x % BH;
+    const int S = p.S, P = p.start_pos, L = p.L;
+    const int ctx = P + S;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int qi = lane & 31, hf = lane >> 5;
+    const int q_row = qb * kPrefillQueriesPerBlock + wave * 32 + qi;
+    const bool q_ok = q_row < S;
+
+    half8 qreg[NC];
+    {
+        const float *qsrc = p.q_rot + ((size_t)bh * S + (q_ok ? q_row : 0)) * D + 8 * hf;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const float4 a = q_ok ? *reinterpret_cast<const float4 *>(qsrc + 16 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 b = q_ok ? *reinterpret_cast<const float4 *>(qsrc + 16 * c + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+            qreg[c][0] = (_Float16)a.x; qreg[c][1] = (_Float16)a.y; qreg[c][2] = (_Float16)a.z; qreg[c][3] = (_Float16)a.w;
+            qreg[c][4] = (_Float16)b.x; qreg[c][5] = (_Float16)b.y; qreg[c][6] = (_Float16)b.z; qreg[c][7] = (_Float16)b.w;
+        }
+    }
+
+    floatx16 ot[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) ot[dt][v] = 0.f;
+    const float scale = p.scale * kLog2e;
+    float m = kMaxFloor * kLog2e, l = 0.f;
+    const _Float16 *Kb = reinterpret_cast<const _Float16 *>(p.k_cache) + (size_t)bh * L * D;
+    const _Float16 *Vb = reinterpret_cast<const _Float16 *>(p.v_cache) + (size_t)bh * L * D;
+
+    for (int k0 = 0; k0 < ctx; k0 += BN) {
+        __syncthreads(); // every wave is done with the previous tile
+        for (int idx = tid; idx < BN * CPR; idx += 256) {
+            { // K: chunk index fastest (coalesced rows), row-major in LDS
+                const int r = idx / CPR, cc = idx % CPR;
+                half8 kx;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) kx[i] = (_Float16)0;
+                if (k0 + r < ctx) kx = *reinterpret_cast<const half8 *>(Kb + (size_t)(k0 + r) * D + cc * 8);
+                *reinterpret_cast<half8 *>(&sK[r][cc * 8]) = kx;
+            }
+            { // V: key index fastest, transposed into LDS (consecutive lanes write consecutive halfs)
+                const int r = idx % BN, cc = idx / BN;
+                half8 vx;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) vx[i] = (_Float16)0;
+                if (k0 + r < ctx) vx = *reinterpret_cast<const half8 *>(Vb + (size_t)(k0 + r) * D + cc * 8);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) sVt[cc * 8 + i][r] = vx[i];
+            }
+        }
+        if constexpr (HAS_MASK) stage_mask_tile(p, sM, qb, k0, ctx, tid, kLog2e);
+        __syncthreads();
+        float mk[16];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+            if constexpr (HAS_MASK) t = *reinterpret_cast<const float4 *>(&sM[wave * 32 + qi][8 * g4 + 4 * hf]);
+            mk[4 * g4 + 0] = t.x; mk[4 * g4 + 1] = t.y; mk[4 * g4 + 2] = t.z; mk[4 * g4 + 3] = t.w;
+        }
+
+        floatx16 st;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) st[v] = 0.f;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const half8 ka = *reinterpret_cast<const half8 *>(&sK[qi][16 * c + 8 * hf]);
+            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[c], st, 0, 0, 0);
+        }
+
+        float sc[16];
+        float mx = m;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int key = k0 + 8 * (v / 4) + 4 * hf + (v % 4);
+            float x = HAS_MASK ? fmaf(st[v], scale, mk[v]) : st[v] * scale;
+            if (key >= ctx) x = -__builtin_inff();
+            sc[v] = x;
+            mx = fmaxf(mx, x);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float alpha = __builtin_amdgcn_exp2f(m - mx);
+        m = mx;
+        l *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) ot[dt][v] *= alpha;
+        half8 pr[2];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const _Float16 e = (_Float16)__builtin_amdgcn_exp2f(sc[v] - m);
+            pr[v / 8][v % 8] = e;
+            l += (float)e; // normalise by the weights actually multiplied in
+        }
+
+        // O^T += V^T P^T, 16 keys per MFMA
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const half4 lo = *reinterpret_cast<const half4 *>(&sVt[32 * dt + qi][16 * u + 4 * hf]);
+                const half4 hi = *reinterpret_cast<const half4 *>(&sVt[32 * dt + qi][16 * u + 8 + 4 * hf]);
+                half8 va;
+                va[0] = lo[0]; va[1] = lo[1]; va[2] = lo[2]; va[3] = lo[3];
+                va[4] = hi[0]; va[5] = hi[1]; va[6] = hi[2]; va[7] = hi[3];
+                ot[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pr[u], ot[dt], 0, 0, 0);
+            }
+    }
+
+    l += __shfl_xor(l, 32);
+    if (q_ok) {
+        float *dst = p.out + ((size_t)bh * S + q_row) * D;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                float4 r;
+                r.x = ot[dt][4 * g4 + 0] / l;
                 r.y = ot[dt][4 * g4 + 1] / l;
                 r.z = ot[dt][4 * g4 + 2] / l;
                 r.w = ot[dt][4 * g4 + 3] / l;

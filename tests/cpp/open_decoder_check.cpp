@@ -275,7 +275,7 @@ template <OperationType Op, typename CacheT> static void runAll(const char *tag)
         std::snprintf(name, sizeof name, "%s prompt forward int8 within one step", tag);
         report(name, worst8 <= 1 && pctx.calls_pre == 1 && pctx.calls_post == 1, worst8);
         std::snprintf(name, sizeof name, "%s prompt forward output scale", tag);
-        report(name, worst_s <= 1e-5, worst_s);
+        report(name, worst_s <= (code ? 1e-3 : 1e-5), worst_s); // half caches: fp16 matrix-core operands
         std::snprintf(name, sizeof name, "%s prompt forward k_cache bit-exact", tag);
         report(name, !std::memcmp(kc_got.data(), kc_ref.data(), kc.size() * sizeof(CacheT)));
         dec.setExternalStages(stages_keep);
