@@ -293,9 +293,10 @@ typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 // kernels.  Contraction slots: a lane-half hf supplies eight consecutive slots of each MFMA; for the
 // first product they are d = 16c + 8hf + r, for the second the keys this lane holds after the first:
 // 16u + 4hf + r (r < 4) and 16u + 8 + 4hf + (r - 4).
-// three waves per SIMD (<= 170 registers, accumulators in VGPRs): 0.56 -> 0.48 ms at B=8, S=1024
+// Two waves per SIMD with the next tile prefetched into registers (244 VGPRs) beat three waves per
+// SIMD without prefetch (168 VGPRs): 0.48 -> 0.47 ms at B=8, S=1024 and 0.82 -> 0.66 ms at B=1, S=4096.
 #ifndef FLATTN_PREFILL_F16_WAVES
-#define FLATTN_PREFILL_F16_WAVES 3
+#define FLATTN_PREFILL_F16_WAVES 2
 #endif
 template <int D, bool HAS_MASK>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(FLATTN_PREFILL_F16_WAVES, 8)))
@@ -344,29 +345,68 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     const _Float16 *Kb = reinterpret_cast<const _Float16 *>(p.k_cache) + (size_t)bh * L * D;
     const _Float16 *Vb = reinterpret_cast<const _Float16 *>(p.v_cache) + (size_t)bh * L * D;
 
-    for (int k0 = 0; k0 < ctx; k0 += BN) {
-        __syncthreads(); // every wave is done with the previous tile
-        for (int idx = tid; idx < BN * CPR; idx += 256) {
-            { // K: chunk index fastest (coalesced rows), row-major in LDS
+    // Tile staging in two halves so that the global loads of tile i+1 fly while tile i is multiplied:
+    // fetch (global -> registers: K and V chunks and the mask tile), commit (registers -> LDS).
+    constexpr int LPT = (BN * CPR + 255) / 256; // 16-byte chunks per thread per tile, for K and for V
+    constexpr int MPT = kPrefillQueriesPerBlock / 8; // mask values per thread per tile
+    half8 kstage[LPT], vstage[LPT];
+    float mstage[HAS_MASK ? MPT : 1];
+    const int mc = tid & 31, mr0 = tid >> 5; // mask tile: 32 consecutive lanes read one 128-byte row segment
+    const int mq0 = qb * kPrefillQueriesPerBlock + mr0;
+    const float *msrc = HAS_MASK ? p.attn_mask + (size_t)(P + mq0) * p.mask_ld + mc : nullptr;
+    const size_t mstep = (size_t)8 * p.mask_ld;
+
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < LPT; ++j) {
+            const int idx = tid + j * 256;
+            { // K: chunk index fastest (coalesced rows)
                 const int r = idx / CPR, cc = idx % CPR;
-                half8 kx;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) kx[i] = (_Float16)0;
-                if (k0 + r < ctx) kx = *reinterpret_cast<const half8 *>(Kb + (size_t)(k0 + r) * D + cc * 8);
-                *reinterpret_cast<half8 *>(&sK[r][cc * 8]) = kx;
+                for (int i = 0; i < 8; ++i) kstage[j][i] = (_Float16)0;
+                if (idx < BN * CPR && k0 + r < ctx)
+                    kstage[j] = *reinterpret_cast<const half8 *>(Kb + (size_t)(k0 + r) * D + cc * 8);
             }
-            { // V: key index fastest, transposed into LDS (consecutive lanes write consecutive halfs)
+            { // V: key index fastest (it is stored transposed)
                 const int r = idx % BN, cc = idx / BN;
-                half8 vx;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) vx[i] = (_Float16)0;
-                if (k0 + r < ctx) vx = *reinterpret_cast<const half8 *>(Vb + (size_t)(k0 + r) * D + cc * 8);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) sVt[cc * 8 + i][r] = vx[i];
+                for (int i = 0; i < 8; ++i) vstage[j][i] = (_Float16)0;
+                if (idx < BN * CPR && k0 + r < ctx)
+                    vstage[j] = *reinterpret_cast<const half8 *>(Vb + (size_t)(k0 + r) * D + cc * 8);
             }
         }
-        if constexpr (HAS_MASK) stage_mask_tile(p, sM, qb, k0, ctx, tid, kLog2e);
+        if constexpr (HAS_MASK) {
+            const bool key_ok = k0 + mc < ctx;
+#pragma unroll
+            for (int j = 0; j < MPT; ++j) {
+                mstage[j] = 0.f;
+                if (key_ok && mq0 + 8 * j < S) mstage[j] = msrc[k0 + j * mstep];
+            }
+        }
+    };
+    auto commit = [&]() {
+#pragma unroll
+        for (int j = 0; j < LPT; ++j) {
+            const int idx = tid + j * 256;
+            if (idx < BN * CPR) {
+                *reinterpret_cast<half8 *>(&sK[idx / CPR][(idx % CPR) * 8]) = kstage[j];
+                const int r = idx % BN, cc = idx / BN;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) sVt[cc * 8 + i][r] = vstage[j][i]; // consecutive lanes, consecutive halfs
+            }
+        }
+        if constexpr (HAS_MASK) {
+#pragma unroll
+            for (int j = 0; j < MPT; ++j) sM[mr0 + 8 * j][mc] = mstage[j] * kLog2e; // pre-scaled for the base-2 softmax
+        }
+    };
+
+    fetch(0);
+    for (int k0 = 0; k0 < ctx; k0 += BN) {
+        __syncthreads(); // every wave is done with the previous tile
+        commit();
         __syncthreads();
+        if (k0 + BN < ctx) fetch(k0 + BN); // in flight during the products below
         float mk[16];
 #pragma unroll
         for (int g4 = 0; g4 < 4; ++g4) {
@@ -395,13 +435,15 @@ void prefill_attn_f16_kernel(const PrefillParams p)
             mx = fmaxf(mx, x);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float alpha = __builtin_amdgcn_exp2f(m - mx);
-        m = mx;
-        l *= alpha;
+        if (__ballot(mx != m) != 0ull) { // wave-uniform: once the maxima have settled alpha is exactly 1
+            const float alpha = __builtin_amdgcn_exp2f(m - mx);
+            m = mx;
+            l *= alpha;
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
+            for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) ot[dt][v] *= alpha;
+                for (int v = 0; v < 16; ++v) ot[dt][v] *= alpha;
+        }
         half8 pr[2];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
