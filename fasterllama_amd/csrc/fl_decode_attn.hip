@@ -483,7 +483,7 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     p.q = io->q; p.k_new = io->k_new; p.v_new = io->v_new;
     p.k_cache = io->k_cache; p.v_cache = io->v_cache;
     p.freq_cis = io->freq_cis; p.attn_mask = io->attn_mask;
-    p.q_rot = reinterpret_cast<float *>(ws + wl.q_rot);
+    p.q_rot = ws + wl.q_rot;
     p.out = io->out ? io->out : reinterpret_cast<float *>(ws + wl.tmp_out);
     p.inp_scale = io->qkv_inp_scale; p.wq_scale = io->q_weight_scale;
     p.wk_scale = io->k_weight_scale; p.wv_scale = io->v_weight_scale;

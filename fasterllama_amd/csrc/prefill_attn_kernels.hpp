@@ -7,11 +7,10 @@
 // Unlike the decode step this is a dense contraction (S x ctx x D per head), so it runs on the
 // matrix cores.  FP32 caches: FP32 MFMA (v_mfma_f32_32x32x2_f32) with FP32 operands, which keeps the
 // 1e-5 parity bar of the FP32 path.  fp16 caches: fp16 MFMA (v_mfma_f32_32x32x16_f16) with FP32
-// accumulation (prefill_attn_f16_kernel); the FP32-MFMA kernel also accepts fp16 caches, widening
-// them when a tile is staged in LDS.
+// accumulation (prefill_attn_f16_kernel).
 //
 // Two kernels:
-//   prefill_rope_append_kernel  elementwise: RoPE(q) -> workspace [B,H,S,D] fp32, RoPE(k), v ->
+//   prefill_rope_append_kernel  elementwise: RoPE(q) -> workspace [B,H,S,D], RoPE(k), v ->
 //                               cache rows start_pos + s (bit-identical to the decode step's rows)
 //   prefill_attn_kernel         flash-attention style: a workgroup owns 128 queries of one (b,h)
 //                               (32 per wave) and walks the keys 32 at a time through LDS.
@@ -29,7 +28,7 @@ struct PrefillParams {
     void *k_cache, *v_cache;       // [B,H,L,D]
     const float *freq_cis;
     const float *attn_mask;
-    float *q_rot; // workspace [B,H,S,D] fp32
+    void *q_rot;  // workspace [B,H,S,D]: fp32 for FP32 caches, fp16 (the MFMA operand type) for fp16 caches
     float *out;   // [B,H,S,D] fp32
     const float *inp_scale, *wq_scale, *wk_scale, *wv_scale;
     int64_t mask_ld;
@@ -65,7 +64,7 @@ __global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillP
     const float inp_scale = is_i32 ? p.inp_scale[bs] : 0.f;
     const size_t in_off = (size_t)row * D;
     const size_t bh = (size_t)b * p.H + h;
-    float *qdst = p.q_rot + (bh * p.S + s) * D;
+    T *qdst = reinterpret_cast<T *>(p.q_rot) + (bh * p.S + s) * D;
     T *kdst = reinterpret_cast<T *>(p.k_cache) + (bh * p.L + pos) * D;
     T *vdst = reinterpret_cast<T *>(p.v_cache) + (bh * p.L + pos) * D;
 
@@ -76,14 +75,14 @@ __global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillP
         load_token_chunk<T, VEC>(p.q, in_off + e0, is_i32, inp_scale, is_i32 ? p.wq_scale + h * D + e0 : nullptr, qx);
         load_token_chunk<T, VEC>(p.k_new, in_off + e0, is_i32, inp_scale, is_i32 ? p.wk_scale + h * D + e0 : nullptr, kx);
         load_token_chunk<T, VEC>(p.v_new, in_off + e0, is_i32, inp_scale, is_i32 ? p.wv_scale + h * D + e0 : nullptr, vx);
-        V kt, vt;
+        V kt, vt, qt;
 #pragma unroll
         for (int i = 0; i < VEC; i += 4) {
             const float4 f = *reinterpret_cast<const float4 *>(freq + e0 + i);
             float4 qo;
             rope_pair(qx[i], qx[i + 1], f.x, f.y, qo.x, qo.y);
             rope_pair(qx[i + 2], qx[i + 3], f.z, f.w, qo.z, qo.w);
-            *reinterpret_cast<float4 *>(qdst + e0 + i) = qo;
+            qt[i] = (T)qo.x; qt[i + 1] = (T)qo.y; qt[i + 2] = (T)qo.z; qt[i + 3] = (T)qo.w;
             float r0, r1, r2, r3;
             rope_pair(kx[i], kx[i + 1], f.x, f.y, r0, r1);
             rope_pair(kx[i + 2], kx[i + 3], f.z, f.w, r2, r3);
@@ -92,6 +91,7 @@ __global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillP
         }
 #pragma unroll
         for (int i = 0; i < VEC; ++i) vt[i] = to_storage<T>(vx[i]);
+        *reinterpret_cast<V *>(qdst + e0) = qt;
         *reinterpret_cast<V *>(kdst + e0) = kt;
         *reinterpret_cast<V *>(vdst + e0) = vt;
     }
@@ -163,7 +163,8 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
 
     float qreg[NC][4];
     {
-        const float *qsrc = p.q_rot + ((size_t)bh * S + (q_ok ? q_row : 0)) * D + 4 * hf;
+        static_assert(std::is_same<T, float>::value, "the FP32-MFMA kernel reads FP32 rotated queries");
+        const float *qsrc = reinterpret_cast<const float *>(p.q_rot) + ((size_t)bh * S + (q_ok ? q_row : 0)) * D + 4 * hf;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             float4 t = q_ok ? *reinterpret_cast<const float4 *>(qsrc + 8 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -325,13 +326,12 @@ void prefill_attn_f16_kernel(const PrefillParams p)
 
     half8 qreg[NC];
     {
-        const float *qsrc = p.q_rot + ((size_t)bh * S + (q_ok ? q_row : 0)) * D + 8 * hf;
+        const _Float16 *qsrc = reinterpret_cast<const _Float16 *>(p.q_rot) + ((size_t)bh * S + (q_ok ? q_row : 0)) * D + 8 * hf;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
-            const float4 a = q_ok ? *reinterpret_cast<const float4 *>(qsrc + 16 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
-            const float4 b = q_ok ? *reinterpret_cast<const float4 *>(qsrc + 16 * c + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-            qreg[c][0] = (_Float16)a.x; qreg[c][1] = (_Float16)a.y; qreg[c][2] = (_Float16)a.z; qreg[c][3] = (_Float16)a.w;
-            qreg[c][4] = (_Float16)b.x; qreg[c][5] = (_Float16)b.y; qreg[c][6] = (_Float16)b.z; qreg[c][7] = (_Float16)b.w;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) qreg[c][i] = (_Float16)0;
+            if (q_ok) qreg[c] = *reinterpret_cast<const half8 *>(qsrc + 16 * c);
         }
     }
 
