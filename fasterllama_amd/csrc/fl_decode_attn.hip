@@ -3,6 +3,7 @@
 // allocation, no synchronisation, no state kept between calls.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdint>
 #include <type_traits>
@@ -36,19 +37,20 @@ inline bool check_hip(hipError_t e)
     return true;
 }
 
-// Compute units of the current device, cached per device id.
+// Compute units of the current device.  The only thing the library remembers between calls: an
+// immutable property of the hardware, cached per device id (256 when no device can be queried).
 int device_cus()
 {
-    static int cached[64] = {0};
+    static std::atomic<int> cached[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cached[dev] == 0) {
-        int n = 0;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
             n = 256;
-        cached[dev] = n;
+        cached[dev].store(n, std::memory_order_relaxed);
     }
-    return cached[dev];
+    return n;
 }
 
 bool head_dim_ok(int D)
@@ -235,17 +237,23 @@ hipError_t dispatch_split(int D, const Params &p, dim3 grid, hipStream_t stream)
 
 bool prefill_head_dim_ok(int D) { return D == 32 || D == 64 || D == 128; }
 
+// Workspace layout of the prompt phase: [rotated queries B*H*S*D] [float output B*H*S*D (used when the
+// caller asks for INT8 only)] [mask tile classes: one word per 128-query block and 32-key tile, sized
+// for a context that fills the cache], each 256-byte aligned.
 struct PrefillWorkspace {
-    size_t q_rot, tmp_out, total;
+    size_t q_rot, tmp_out, tile_class, total;
 };
 
 PrefillWorkspace prefill_workspace(const fl_attn_desc *d, int S)
 {
     const size_t n = align_up((size_t)d->batch_size * d->head_num * (size_t)S * d->size_per_head * sizeof(float), 256);
+    const size_t qblocks = ((size_t)S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock;
+    const size_t ktiles = ((size_t)d->total_len + flattn::kPrefillKeysPerStep - 1) / flattn::kPrefillKeysPerStep;
     PrefillWorkspace w;
     w.q_rot = 0;
     w.tmp_out = n;
-    w.total = 2 * n;
+    w.tile_class = 2 * n;
+    w.total = w.tile_class + align_up(qblocks * ktiles * sizeof(uint32_t), 256);
     return w;
 }
 
@@ -263,9 +271,14 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
     const unsigned qblocks = (unsigned)((p.S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock);
     const dim3 grid(qblocks * (unsigned)(p.B * p.H)); // (b,h) fastest: the query blocks of one head share an XCD's L2
     if constexpr (std::is_same<T, _Float16>::value) {
-        if (p.attn_mask)
+        if (p.attn_mask) {
+            const int ktiles = (p.start_pos + p.S + flattn::kPrefillKeysPerStep - 1) / flattn::kPrefillKeysPerStep;
+            hipLaunchKernelGGL(flattn::prefill_mask_classify_kernel, dim3((unsigned)ktiles, qblocks), dim3(256), 0, stream, p,
+                               ktiles);
+            e = hipGetLastError();
+            if (e != hipSuccess) return e;
             hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, true>), grid, dim3(256), 0, stream, p);
-        else
+        } else
             hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, false>), grid, dim3(256), 0, stream, p);
     } else {
         if (p.attn_mask)
@@ -302,7 +315,8 @@ const char *fl_attn_strerror(int status)
     switch (status) {
     case FL_ATTN_OK: return "ok";
     case FL_ATTN_ERR_NULL_POINTER: return "a required pointer is NULL";
-    case FL_ATTN_ERR_HEAD_DIM: return "invalid size_per_head (supported: 32, 64, 128, 256, 512, 1024)";
+    case FL_ATTN_ERR_HEAD_DIM:
+        return "invalid size_per_head (decode step: 32, 64, 128, 256, 512, 1024; prompt phase: 32, 64, 128)";
     case FL_ATTN_ERR_SHAPE: return "invalid batch_size / head_num / total_len";
     case FL_ATTN_ERR_POSITION: return "start_pos or rope_row out of range for total_len";
     case FL_ATTN_ERR_WORKSPACE: return "workspace missing, too small or not 256-byte aligned";
@@ -484,6 +498,7 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     p.k_cache = io->k_cache; p.v_cache = io->v_cache;
     p.freq_cis = io->freq_cis; p.attn_mask = io->attn_mask;
     p.q_rot = ws + wl.q_rot;
+    p.tile_class = reinterpret_cast<uint32_t *>(ws + wl.tile_class);
     p.out = io->out ? io->out : reinterpret_cast<float *>(ws + wl.tmp_out);
     p.inp_scale = io->qkv_inp_scale; p.wq_scale = io->q_weight_scale;
     p.wk_scale = io->k_weight_scale; p.wv_scale = io->v_weight_scale;

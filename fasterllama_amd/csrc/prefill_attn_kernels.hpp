@@ -29,6 +29,7 @@ struct PrefillParams {
     const float *freq_cis;
     const float *attn_mask;
     void *q_rot;  // workspace [B,H,S,D]: fp32 for FP32 caches, fp16 (the MFMA operand type) for fp16 caches
+    uint32_t *tile_class; // workspace [ceil(S/128), ceil((start_pos+S)/32)]: mask tile classes (fp16 caches with a mask)
     float *out;   // [B,H,S,D] fp32
     const float *inp_scale, *wq_scale, *wk_scale, *wv_scale;
     int64_t mask_ld;
@@ -104,30 +105,6 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 constexpr int kPrefillQueriesPerBlock = 128; // 4 waves x 32 queries
 constexpr int kPrefillKeysPerStep = 32;
 constexpr int kMaskTileLd = kPrefillKeysPerStep + 4; // padded: 128-bit reads of 8 consecutive rows hit 32 banks
-
-// Stages the additive-mask tile of a workgroup (128 queries x 32 keys, rows start_pos + q of the
-// caller's [*, mask_ld] matrix) in LDS with coalesced loads: 256 cache-line reads per tile, where
-// per-lane gathers (each lane a different mask row) cost 4096 and made the texture path the bottleneck
-// of the fp16 kernel.  Entries outside the prompt or the context are 0 (their scores are forced to
-// -inf or never used).  `mul` pre-scales the mask for the base-2 softmax.
-__device__ __forceinline__ void stage_mask_tile(const PrefillParams &p, float (*sM)[kMaskTileLd], int qb, int k0, int ctx,
-                                                int tid, float mul)
-{
-    // thread -> (row r0 + 8j, column c): 32 consecutive lanes read one 128-byte row segment
-    const int c = tid & 31, r0 = tid >> 5;
-    const int q0 = qb * kPrefillQueriesPerBlock + r0;
-    const bool key_ok = k0 + c < ctx;
-    const float *src = p.attn_mask + (size_t)(p.start_pos + q0) * p.mask_ld + k0 + c;
-    const size_t step = (size_t)8 * p.mask_ld;
-    float x[kPrefillQueriesPerBlock / 8];
-#pragma unroll
-    for (int j = 0; j < kPrefillQueriesPerBlock / 8; ++j) { // all 16 loads in flight together
-        x[j] = 0.f;
-        if (key_ok && q0 + 8 * j < p.S) x[j] = src[j * step];
-    }
-#pragma unroll
-    for (int j = 0; j < kPrefillQueriesPerBlock / 8; ++j) sM[r0 + 8 * j][c] = x[j] * mul;
-}
 
 // MFMA operand layouts used below (v_mfma_f32_32x32x2_f32, D += A(32x2) * B(2x32)):
 //   A: lane holds A[row = lane % 32][k = lane / 32];  B: lane holds B[k = lane / 32][col = lane % 32];
@@ -281,48 +258,154 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
     }
 }
 
+// ---------------------------------------------------------------- mask tile classes
+
+// The additive mask is caller data, but the masks that occur in practice are piecewise trivial: a
+// causal mask is all zero below the diagonal band and all "minus huge" above it.  A small kernel
+// classifies every 32-query x 32-key tile of the mask rows this call uses, once per call (the mask
+// is shared by all (b,h)), and the fp16 attention kernel then
+//   SKIP   never touches a tile whose entries are all <= -1e30: with finite K the scores
+//          v = s*scale + mask stay below every running maximum (floor -1e9) and exp(v - max) is
+//          exactly 0, so the tile contributes exact zeros to the sum and the output — skipping it
+//          is bit-identical to evaluating it (decoder_kernels.cu:811-833 arithmetic);
+//   ZERO   drops the mask term where all entries are +-0;
+//   MIXED  evaluates the general form.
+// One 32-bit word per (128-query block, key tile): byte w is the class of the block's w-th wave.
+constexpr uint32_t kTileSkip = 0, kTileZero = 1, kTileMixed = 2;
+constexpr float kMaskedBelow = -1e30f;
+constexpr float kLazyMax = 8.0f; // base-2 units
+
+// grid = (key tiles, query blocks), block = 256.
+__global__ __launch_bounds__(256) void prefill_mask_classify_kernel(const PrefillParams p, int NT)
+{
+    __shared__ uint32_t s_cls[4];
+    const int t = blockIdx.x, qb = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int ctx = p.start_pos + p.S;
+    const int q0 = qb * kPrefillQueriesPerBlock + wave * 32;
+    uint32_t cls = kTileSkip; // a wave whose queries are all beyond the prompt has nothing to do
+    if (q0 < p.S) {
+        // entries beyond the prompt or the context repeat the last valid row / column: neutral for both tests
+        const int col = min(t * kPrefillKeysPerStep + (lane & 31), ctx - 1);
+        uint32_t nonzero = 0;
+        bool open = false;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int q = min(q0 + 2 * j + (lane >> 5), p.S - 1);
+            const float v = p.attn_mask[(size_t)(p.start_pos + q) * p.mask_ld + col];
+            nonzero |= __float_as_uint(v) << 1; // the sign is shifted out: -0 counts as zero
+            open |= !(v <= kMaskedBelow);       // a NaN entry keeps the tile
+        }
+        cls = __ballot(open) == 0ull ? kTileSkip : (__ballot(nonzero != 0u) == 0ull ? kTileZero : kTileMixed);
+    }
+    if (lane == 0) s_cls[wave] = cls;
+    __syncthreads();
+    if (tid == 0) p.tile_class[(size_t)qb * NT + t] = s_cls[0] | (s_cls[1] << 8) | (s_cls[2] << 16) | (s_cls[3] << 24);
+}
+
 // ---------------------------------------------------------------- fp16 caches: fp16 MFMA
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float2v __attribute__((ext_vector_type(2)));
+
+// max over both 32-lane halves of a wave, in every lane: one v_permlane32_swap (the upper half of
+// the first operand trades places with the lower half of the second) and one v_max.
+__device__ __forceinline__ float cross_half_max(float x)
+{
+    const unsigned u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lanes 4j..4j+3 address 16 consecutive halfs of
+// matrix row j (j < 4, four halfs per lane) and lane i receives element i of rows 0, 1, 2, 3.
+typedef short short4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ half4 lds_read_tr16(const _Float16 *lds)
+{
+    typedef short4v __attribute__((address_space(3))) * lds_ptr;
+    return __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)lds));
+}
+
+__device__ __forceinline__ float max16(const floatx16 &a)
+{
+    float r = fmaxf(fmaxf(a[0], a[1]), a[2]); // pairs of fmaxf fold into v_max3_f32
+#pragma unroll
+    for (int v = 3; v < 15; v += 2) r = fmaxf(fmaxf(r, a[v]), a[v + 1]);
+    return fmaxf(r, a[15]);
+}
 
 // Same algorithm as prefill_attn_kernel for fp16 caches, on v_mfma_f32_32x32x16_f16: K and V tiles
-// stay fp16 in LDS (V transposed, so a lane fetches the eight keys of one MFMA as two 64-bit reads),
-// rotated queries and probabilities are rounded to fp16 as MFMA operands, every accumulation is
-// FP32 (scores, softmax statistics, output).  The rounding of q and p costs ~1e-4 absolute on the
-// output, inside the 2e-3 bar of the fp16 path.  The softmax runs in base 2 like the fp16 decode
-// kernels.  Contraction slots: a lane-half hf supplies eight consecutive slots of each MFMA; for the
-// first product they are d = 16c + 8hf + r, for the second the keys this lane holds after the first:
-// 16u + 4hf + r (r < 4) and 16u + 8 + 4hf + (r - 4).
-// Two waves per SIMD with the next tile prefetched into registers (244 VGPRs) beat three waves per
-// SIMD without prefetch (168 VGPRs): 0.48 -> 0.47 ms at B=8, S=1024 and 0.82 -> 0.66 ms at B=1, S=4096.
-#ifndef FLATTN_PREFILL_F16_WAVES
-#define FLATTN_PREFILL_F16_WAVES 2
-#endif
+// stay fp16 in LDS, rotated queries and probabilities are rounded to fp16 as MFMA operands, every
+// accumulation is FP32 (scores, softmax statistics, output).  The rounding of q and p costs ~1e-4
+// absolute on the output, inside the 2e-3 bar of the fp16 path.  The softmax runs in base 2 like the
+// fp16 decode kernels.
+//
+// The matrix cores need 512 cycles per wave and 32x32 tile at D = 128; the softmax between the two
+// products runs on the vector ALU of the same SIMD at 4 cycles per instruction, so its instruction
+// count per score decides the speed (two waves per SIMD overlap one wave's softmax with the other's
+// MFMAs).  Per score the common tile costs: 1/2 v_max3 (maximum over the raw products; the scale is
+// positive, so it commutes with max), 1 v_fma (s*scale - m), 1 v_exp, 1/2 v_cvt_pk_f16_f32 and
+// 1/2 v_dot2c_f32_f16 (the row sum, taken over the rounded probabilities that are multiplied in).
+//
+// Data path: K and V tiles (32 keys) are double-buffered in LDS, row-major with padded rows; loads of
+// tile t+2 are in flight in registers while tile t is multiplied, one barrier per tile.  The first
+// product reads K rows as 128-bit operands (S^T = K Q^T).  The second, O^T = V^T P^T, needs eight
+// keys of one d per lane: ds_read_b64_tr_b16 delivers exactly that from the row-major tile (within
+// 16 lanes, lanes 4j..4j+3 address 16 consecutive halfs of row j; lane i receives element i of rows
+// 0..3), so V is never transposed in memory.  Contraction slots of the second product: a lane-half
+// hf holds the keys 16u + 4hf + r (r < 4) and 16u + 8 + 4hf + (r - 4) after the first.
+//
+// With a mask, tiles are processed according to their class (see above); tiles that every wave of
+// the workgroup skips are not even loaded.
 template <int D, bool HAS_MASK>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(FLATTN_PREFILL_F16_WAVES, 8)))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8)))
 void prefill_attn_f16_kernel(const PrefillParams p)
 {
     constexpr int BN = kPrefillKeysPerStep; // 32
-    constexpr int LDK = D + 8;              // halfs; rows start 4 banks apart
-    constexpr int LDV = BN + 4;             // halfs; 18-dword rows: 16 lanes x 64-bit reads hit 32 distinct banks
+    constexpr int LDK = D + 8;              // halfs; rows start 4 banks apart (128-bit operand reads)
+    constexpr int LDV = D + 32;             // halfs; rows start 16 banks apart (8 rows x 64 bytes per transposing read)
     constexpr int NC = D / 16;
     constexpr int NDT = D / 32;
     constexpr int CPR = D / 8; // 16-byte chunks per cache row
+    constexpr int LPT = (BN * CPR + 255) / 256; // chunks per thread per tile, for K and for V
     static_assert(D % 32 == 0, "head size must be a multiple of 32");
 
-    __shared__ __attribute__((aligned(16))) _Float16 sK[BN][LDK];
-    __shared__ __attribute__((aligned(16))) _Float16 sVt[D][LDV];
-    __shared__ float sM[HAS_MASK ? kPrefillQueriesPerBlock : 1][kMaskTileLd];
+    __shared__ __attribute__((aligned(16))) _Float16 sK[2][BN][LDK];
+    __shared__ __attribute__((aligned(16))) _Float16 sV[2][BN][LDV];
+    __shared__ __attribute__((aligned(16))) float sM[HAS_MASK ? kPrefillQueriesPerBlock : 1][kMaskTileLd];
+    __shared__ int s_end;
 
     const int BH = p.B * p.H;
     const int qb = blockIdx.x / BH, bh = blockIdx.x % BH;
     const int S = p.S, P = p.start_pos, L = p.L;
     const int ctx = P + S;
+    const int NT = (ctx + BN - 1) / BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int qi = lane & 31, hf = lane >> 5;
     const int q_row = qb * kPrefillQueriesPerBlock + wave * 32 + qi;
     const bool q_ok = q_row < S;
+
+    // last tile any wave of this workgroup needs
+    const uint32_t *cls = HAS_MASK ? p.tile_class + (size_t)qb * NT : nullptr;
+    int t_end = NT;
+    if constexpr (HAS_MASK) {
+        if (tid == 0) s_end = 0;
+        __syncthreads();
+        int last = 0;
+        for (int t = tid; t < NT; t += 256)
+            if (cls[t] != 0u) last = t + 1;
+        if (last > 0) atomicMax(&s_end, last);
+        __syncthreads();
+        t_end = s_end;
+    }
+    auto next_tile = [&](int t) { // uniform: the next tile some wave needs, or t_end
+        ++t;
+        if constexpr (HAS_MASK)
+            while (t < t_end && cls[t] == 0u) ++t;
+        return t;
+    };
 
     half8 qreg[NC];
     {
@@ -345,125 +428,169 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     const _Float16 *Kb = reinterpret_cast<const _Float16 *>(p.k_cache) + (size_t)bh * L * D;
     const _Float16 *Vb = reinterpret_cast<const _Float16 *>(p.v_cache) + (size_t)bh * L * D;
 
-    // Tile staging in two halves so that the global loads of tile i+1 fly while tile i is multiplied:
-    // fetch (global -> registers: K and V chunks and the mask tile), commit (registers -> LDS).
-    constexpr int LPT = (BN * CPR + 255) / 256; // 16-byte chunks per thread per tile, for K and for V
-    constexpr int MPT = kPrefillQueriesPerBlock / 8; // mask values per thread per tile
+    // global -> registers (fetch) and registers -> LDS (commit) of one key tile
     half8 kstage[LPT], vstage[LPT];
-    float mstage[HAS_MASK ? MPT : 1];
-    const int mc = tid & 31, mr0 = tid >> 5; // mask tile: 32 consecutive lanes read one 128-byte row segment
-    const int mq0 = qb * kPrefillQueriesPerBlock + mr0;
-    const float *msrc = HAS_MASK ? p.attn_mask + (size_t)(P + mq0) * p.mask_ld + mc : nullptr;
-    const size_t mstep = (size_t)8 * p.mask_ld;
-
-    auto fetch = [&](int k0) {
+    constexpr bool EXACT = (BN * CPR) % 256 == 0; // every thread owns LPT chunks of each matrix
+    auto fetch = [&](int t) {
+        const int k0 = t * BN;
+        const bool tail = k0 + BN > ctx;
 #pragma unroll
         for (int j = 0; j < LPT; ++j) {
             const int idx = tid + j * 256;
-            { // K: chunk index fastest (coalesced rows)
-                const int r = idx / CPR, cc = idx % CPR;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) kstage[j][i] = (_Float16)0;
-                if (idx < BN * CPR && k0 + r < ctx)
+            const int r = idx / CPR, cc = idx % CPR;
+            if (!tail) {
+                if (EXACT || idx < BN * CPR) {
                     kstage[j] = *reinterpret_cast<const half8 *>(Kb + (size_t)(k0 + r) * D + cc * 8);
-            }
-            { // V: key index fastest (it is stored transposed)
-                const int r = idx % BN, cc = idx / BN;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) vstage[j][i] = (_Float16)0;
-                if (idx < BN * CPR && k0 + r < ctx)
                     vstage[j] = *reinterpret_cast<const half8 *>(Vb + (size_t)(k0 + r) * D + cc * 8);
-            }
-        }
-        if constexpr (HAS_MASK) {
-            const bool key_ok = k0 + mc < ctx;
+                }
+            } else { // rows beyond the context may hold anything: they enter as zeros
 #pragma unroll
-            for (int j = 0; j < MPT; ++j) {
-                mstage[j] = 0.f;
-                if (key_ok && mq0 + 8 * j < S) mstage[j] = msrc[k0 + j * mstep];
+                for (int i = 0; i < 8; ++i) kstage[j][i] = vstage[j][i] = (_Float16)0;
+                if ((EXACT || idx < BN * CPR) && k0 + r < ctx) {
+                    kstage[j] = *reinterpret_cast<const half8 *>(Kb + (size_t)(k0 + r) * D + cc * 8);
+                    vstage[j] = *reinterpret_cast<const half8 *>(Vb + (size_t)(k0 + r) * D + cc * 8);
+                }
             }
         }
     };
-    auto commit = [&]() {
+    auto commit = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < LPT; ++j) {
             const int idx = tid + j * 256;
-            if (idx < BN * CPR) {
-                *reinterpret_cast<half8 *>(&sK[idx / CPR][(idx % CPR) * 8]) = kstage[j];
-                const int r = idx % BN, cc = idx / BN;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) sVt[cc * 8 + i][r] = vstage[j][i]; // consecutive lanes, consecutive halfs
+            if (EXACT || idx < BN * CPR) {
+                *reinterpret_cast<half8 *>(&sK[buf][idx / CPR][(idx % CPR) * 8]) = kstage[j];
+                *reinterpret_cast<half8 *>(&sV[buf][idx / CPR][(idx % CPR) * 8]) = vstage[j];
             }
-        }
-        if constexpr (HAS_MASK) {
-#pragma unroll
-            for (int j = 0; j < MPT; ++j) sM[mr0 + 8 * j][mc] = mstage[j] * kLog2e; // pre-scaled for the base-2 softmax
         }
     };
 
-    fetch(0);
-    for (int k0 = 0; k0 < ctx; k0 += BN) {
-        __syncthreads(); // every wave is done with the previous tile
-        commit();
-        __syncthreads();
-        if (k0 + BN < ctx) fetch(k0 + BN); // in flight during the products below
-        float mk[16];
-#pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-            float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-            if constexpr (HAS_MASK) t = *reinterpret_cast<const float4 *>(&sM[wave * 32 + qi][8 * g4 + 4 * hf]);
-            mk[4 * g4 + 0] = t.x; mk[4 * g4 + 1] = t.y; mk[4 * g4 + 2] = t.z; mk[4 * g4 + 3] = t.w;
-        }
+    // per-lane source of the transposing V reads: row 4hf + (lane%16)/4, halfs 16*((lane/16)%2) + 4*(lane%4)
+    const int vrow = 4 * hf + ((lane & 15) >> 2), vcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    const float inv_scale = 1.0f / p.scale;
 
-        floatx16 st;
+    // The rotated queries must have landed before the loop: a wait inside it would also wait for
+    // the tile prefetches that are meant to stay in flight.
 #pragma unroll
-        for (int v = 0; v < 16; ++v) st[v] = 0.f;
-#pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            const half8 ka = *reinterpret_cast<const half8 *>(&sK[qi][16 * c + 8 * hf]);
-            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[c], st, 0, 0, 0);
-        }
+    for (int c = 0; c < NC; ++c) asm volatile("" : "+v"(qreg[c]));
 
-        float sc[16];
-        float mx = m;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int key = k0 + 8 * (v / 4) + 4 * hf + (v % 4);
-            float x = HAS_MASK ? fmaf(st[v], scale, mk[v]) : st[v] * scale;
-            if (key >= ctx) x = -__builtin_inff();
-            sc[v] = x;
-            mx = fmaxf(mx, x);
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        if (__ballot(mx != m) != 0ull) { // wave-uniform: once the maxima have settled alpha is exactly 1
-            const float alpha = __builtin_amdgcn_exp2f(m - mx);
-            m = mx;
-            l *= alpha;
-#pragma unroll
-            for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) ot[dt][v] *= alpha;
-        }
-        half8 pr[2];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const _Float16 e = (_Float16)__builtin_amdgcn_exp2f(sc[v] - m);
-            pr[v / 8][v % 8] = e;
-            l += (float)e; // normalise by the weights actually multiplied in
-        }
-
-        // O^T += V^T P^T, 16 keys per MFMA
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const half4 lo = *reinterpret_cast<const half4 *>(&sVt[32 * dt + qi][16 * u + 4 * hf]);
-                const half4 hi = *reinterpret_cast<const half4 *>(&sVt[32 * dt + qi][16 * u + 8 + 4 * hf]);
-                half8 va;
-                va[0] = lo[0]; va[1] = lo[1]; va[2] = lo[2]; va[3] = lo[3];
-                va[4] = hi[0]; va[5] = hi[1]; va[6] = hi[2]; va[7] = hi[3];
-                ot[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pr[u], ot[dt], 0, 0, 0);
+    // Software pipeline over the tiles this workgroup needs: tile t in LDS buffer `buf`, tile t1 in
+    // registers, the loads of tile t2 issued before tile t is multiplied.
+    int t = next_tile(-1);
+    if (t < t_end) {
+        fetch(t);
+        commit(0);
+        int t1 = next_tile(t);
+        if (t1 < t_end) fetch(t1);
+        int buf = 0;
+        while (true) {
+            __syncthreads(); // tile t is visible; every wave is done with the other buffer
+            int t2 = t_end;
+            if (t1 < t_end) {
+                commit(buf ^ 1);
+                t2 = next_tile(t1);
+                if (t2 < t_end) fetch(t2);
             }
+
+            const int k0 = t * BN;
+            uint32_t tc = kTileZero;
+            if constexpr (HAS_MASK) tc = __builtin_amdgcn_readfirstlane((cls[t] >> (8 * wave)) & 0xffu);
+            if (tc != kTileSkip) {
+                // The additive term enters as the initial value of the score accumulator, in units of
+                // the raw product: (s + mask/scale)*scale.  Zero for most tiles; the mask tile where it
+                // is mixed; -inf for keys beyond the context.
+                floatx16 st;
+                const half8 ka0 = *reinterpret_cast<const half8 *>(&sK[buf][qi][8 * hf]);
+                if (k0 + BN > ctx || tc == kTileMixed) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) st[v] = 0.f;
+                    if constexpr (HAS_MASK) {
+                        if (tc == kTileMixed) {
+                            // this wave's 32 mask rows, coalesced (32 lanes read one 128-byte row segment), then
+                            // through the wave's own LDS rows into the score layout
+                            const int col = min(k0 + qi, ctx - 1);
+                            float mraw[16];
+#pragma unroll
+                            for (int j = 0; j < 16; ++j) {
+                                const int q = min(qb * kPrefillQueriesPerBlock + wave * 32 + 2 * j + hf, S - 1);
+                                mraw[j] = p.attn_mask[(size_t)(P + q) * p.mask_ld + col];
+                            }
+#pragma unroll
+                            for (int j = 0; j < 16; ++j) sM[wave * 32 + 2 * j + hf][qi] = mraw[j] * inv_scale;
+                            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                            __builtin_amdgcn_wave_barrier();
+                            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+                            for (int g4 = 0; g4 < 4; ++g4) {
+                                const float4 x = *reinterpret_cast<const float4 *>(&sM[wave * 32 + qi][8 * g4 + 4 * hf]);
+                                st[4 * g4 + 0] = x.x; st[4 * g4 + 1] = x.y; st[4 * g4 + 2] = x.z; st[4 * g4 + 3] = x.w;
+                            }
+                            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                            __builtin_amdgcn_wave_barrier(); // the rows are rewritten by this wave's next mixed tile
+                        }
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        if (k0 + 8 * (v / 4) + 4 * hf + (v % 4) >= ctx) st[v] = -__builtin_inff();
+                    st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka0, qreg[0], st, 0, 0, 0);
+                } else {
+                    floatx16 zero;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) zero[v] = 0.f;
+                    st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka0, qreg[0], zero, 0, 0, 0); // the literal 0 operand
+                }
+#pragma unroll
+                for (int c = 1; c < NC; ++c) {
+                    const half8 ka = *reinterpret_cast<const half8 *>(&sK[buf][qi][16 * c + 8 * hf]);
+                    st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[c], st, 0, 0, 0);
+                }
+
+                // Softmax update of this lane's query (decoder_kernels.cu:811-833 in base 2).  The reference
+                // maximum m may lag the true running maximum by up to kLazyMax (weights up to 2^kLazyMax,
+                // well inside fp16 and exact in the final ratio): with 32 queries per wave some maximum
+                // moves in almost every tile, and rescaling 64 accumulators each time would cost as much
+                // vector time as the softmax itself.
+                const float mx = fmaxf(m, cross_half_max(max16(st)) * scale);
+                if (__ballot(mx > m + kLazyMax) != 0ull) { // wave-uniform
+                    const float alpha = __builtin_amdgcn_exp2f(m - mx);
+                    m = mx;
+                    l *= alpha;
+#pragma unroll
+                    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) ot[dt][v] *= alpha;
+                }
+                const float nm = -m;
+                half8 pr[2];
+#pragma unroll
+                for (int v = 0; v < 16; v += 2) {
+                    float2v e;
+                    e[0] = __builtin_amdgcn_exp2f(fmaf(st[v], scale, nm));
+                    e[1] = __builtin_amdgcn_exp2f(fmaf(st[v + 1], scale, nm));
+                    const half2v h = __builtin_convertvector(e, half2v);
+                    pr[v / 8][v % 8] = h[0];
+                    pr[v / 8][v % 8 + 1] = h[1];
+                    l = __builtin_amdgcn_fdot2(h, half2v{(_Float16)1, (_Float16)1}, l, false); // the weights actually multiplied in
+                }
+
+                // O^T += V^T P^T, 16 keys per MFMA
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        const half4 lo = lds_read_tr16(&sV[buf][16 * u + vrow][32 * dt + vcol]);
+                        const half4 hi = lds_read_tr16(&sV[buf][16 * u + 8 + vrow][32 * dt + vcol]);
+                        half8 va;
+                        va[0] = lo[0]; va[1] = lo[1]; va[2] = lo[2]; va[3] = lo[3];
+                        va[4] = hi[0]; va[5] = hi[1]; va[6] = hi[2]; va[7] = hi[3];
+                        ot[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pr[u], ot[dt], 0, 0, 0);
+                    }
+            }
+
+            if (t1 >= t_end) break;
+            t = t1;
+            t1 = t2;
+            buf ^= 1;
+        }
     }
 
     l += __shfl_xor(l, 32);
