@@ -78,14 +78,18 @@ def bench_prefill(args) -> int:
     k_h = synth.normal((B, S, H, D), np_dt, synth.TENSOR_K_NEW, args.seed)
     v_h = synth.normal((B, S, H, D), np_dt, synth.TENSOR_V_NEW, args.seed)
     freq_h = synth.freq_cis_table(L, D)
-    mask_h = np.where(np.arange(L)[None, :] > np.arange(L)[:, None], -1e5, 0.0).astype(np.float32)  # causal
+    # causal additive mask: masked entries hold -FLT_MAX as in the reference's driver
+    # (samples/llama_fp16.cu:73-81), or -1e5 as in its kernel harness (samples/test.cu:427-437)
+    masked = -1e5 if args.prefill_mask == "causal-1e5" else -float(np.finfo(np.float32).max)
+    blk = 128 if args.prefill_mask == "block-causal" else 1  # block-causal: whole 128-token blocks see each other
+    mask_h = np.where(np.arange(L)[None, :] // blk > np.arange(L)[:, None] // blk, masked, 0.0).astype(np.float32)
     t = lambda a: torch.from_numpy(a).to(dev)
     q, k, v, freq, mask = t(q_h), t(k_h), t(v_h), t(freq_h), t(mask_h)
     kc = torch.zeros(B, H, L, D, dtype=t_dt, device=dev)
     vc = torch.zeros_like(kc)
     out = torch.empty(B, H, S, D, dtype=torch.float32, device=dev)
     op = PrefillAttention(B, H, D, L, S, t_dt, device=dev)
-    io = op.make_io(q, k, v, kc, vc, freq, out, start_pos=P, attn_mask=mask if args.prefill_mask == "causal" else None)
+    io = op.make_io(q, k, v, kc, vc, freq, out, start_pos=P, attn_mask=None if args.prefill_mask == "none" else mask)
     stream = torch.cuda.current_stream(dev)
 
     def run(n):
@@ -103,7 +107,17 @@ def bench_prefill(args) -> int:
     e1.record(stream)
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
-    flops = 4.0 * B * H * S * (P + S) * D  # every query against every key: the mask is generic, nothing is skipped
+    dense_flops = 4.0 * B * H * S * (P + S) * D  # every query against every key
+    # FLOPs the kernels execute: the fp16 kernel drops 32x32 tiles whose mask entries are all <= -1e30 (their
+    # weights are exactly 0); everything else, and the FP32 kernel always, multiplies every tile.
+    flops = dense_flops
+    if w["dtype"] == "f16" and args.prefill_mask != "none":
+        rows = mask_h[P:P + S, :P + S]
+        pad_q, pad_k = (-S) % 32, (-(P + S)) % 32
+        tiles = np.pad(rows, ((0, pad_q), (0, pad_k)), constant_values=-np.inf)
+        tiles = tiles.reshape(tiles.shape[0] // 32, 32, tiles.shape[1] // 32, 32)
+        open_tiles = int(((tiles > -1e30) | np.isnan(tiles)).any(axis=(1, 3)).sum())
+        flops = 4.0 * B * H * open_tiles * 32 * 32 * D
     tflops = flops / (ms * 1e-3) / 1e12
     peak = MFMA_FP16_PEAK_TFLOPS if w["dtype"] == "f16" else MFMA_FP32_PEAK_TFLOPS
 
@@ -117,10 +131,10 @@ def bench_prefill(args) -> int:
         nthreads = max(1, min(16, os.cpu_count() or 1))
         t1 = time.perf_counter()
         want = ref.prefill_attn(q_h[:nb], k_h[:nb], v_h[:nb], kc_s, vc_s, freq_h, start_pos=P,
-                                attn_mask=mask_h if args.prefill_mask == "causal" else None, threads=nthreads)
+                                attn_mask=None if args.prefill_mask == "none" else mask_h, threads=nthreads)
         dt_cpu = time.perf_counter() - t1
         max_err = float(np.abs(out[:nb].cpu().numpy() - want).max())
-        cpu = {"value": round(4.0 * nb * H * S * (P + S) * D / dt_cpu / 1e12, 5), "unit": "TFLOP/s", "cores": nthreads,
+        cpu = {"value": round(4.0 * nb * H * S * (P + S) * D / dt_cpu / 1e12, 5), "unit": "TFLOP/s (dense count)", "cores": nthreads,
                "kind": "port", "sample": f"first {nb} of {B} sequences, scalar oracle with OpenMP over heads, {dt_cpu:.2f} s",
                "gpu_vs_oracle_max_abs_err": max_err}
     print(json.dumps({
@@ -130,8 +144,12 @@ def bench_prefill(args) -> int:
         "dtype": "f16 MFMA, f32 accumulate (f16 storage)" if w["dtype"] == "f16" else "f32 MFMA",
         "data": "synthetic (seeded splitmix64 + Box-Muller N(0,1), seed %d)" % args.seed,
         "config": {"workload": f"{args.workload}: B={B} H={H} D={D} S={S} start_pos={P} L={L} {w['dtype']} KV cache, "
-                               + ("causal additive mask (nothing skipped)" if args.prefill_mask == "causal" else "no mask"),
-                   "flops_per_step": flops},
+                               + {"causal": "causal additive mask, -FLT_MAX above the diagonal",
+                                  "causal-1e5": "causal additive mask, -1e5 above the diagonal",
+                                  "block-causal": "additive mask, causal over blocks of 128 tokens, -FLT_MAX above",
+                                  "none": "no mask"}[args.prefill_mask],
+                   "flops_per_step": flops, "dense_flops_per_step": dense_flops,
+                   "tokens_per_s": round(B * S / (ms * 1e-3), 1)},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(tflops / peak, 4), "traffic": None,
                      "kernel": "prefill_attn_kernel (+ prefill_rope_append_kernel, same step)"},
@@ -171,8 +189,9 @@ def main() -> int:
                     help="only run a plain 1 GiB -> 1 GiB elementwise copy kernel a few times (for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings), then exit")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
-    ap.add_argument("--prefill-mask", default="causal", choices=["causal", "none"],
-                    help="prompt-phase workloads: additive causal mask (as the reference passes) or no mask")
+    ap.add_argument("--prefill-mask", default="causal", choices=["causal", "causal-1e5", "block-causal", "none"],
+                    help="prompt-phase workloads: additive causal mask with -FLT_MAX (the reference's driver) or "
+                         "-1e5 (its kernel harness) above the diagonal, or no mask")
     ap.add_argument("--segment", default="attention", choices=["attention", "int32-int8"],
                     help="attention: q/k/v in the cache dtype -> float output (the headline metric). "
                          "int32-int8: the whole reference segment, int32 GEMM accumulators + scales in, "

@@ -269,7 +269,7 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const unsigned qblocks = (unsigned)((p.S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock);
-    const dim3 grid(qblocks * (unsigned)(p.B * p.H)); // (b,h) fastest: the query blocks of one head share an XCD's L2
+    const dim3 grid(qblocks * (unsigned)(p.B * p.H)); // mapped to (query block, head) by prefill_block_to_tile
     if constexpr (std::is_same<T, _Float16>::value) {
         if (p.attn_mask) {
             const int ktiles = (p.start_pos + p.S + flattn::kPrefillKeysPerStep - 1) / flattn::kPrefillKeysPerStep;

@@ -106,6 +106,27 @@ constexpr int kPrefillQueriesPerBlock = 128; // 4 waves x 32 queries
 constexpr int kPrefillKeysPerStep = 32;
 constexpr int kMaskTileLd = kPrefillKeysPerStep + 4; // padded: 128-bit reads of 8 consecutive rows hit 32 banks
 
+// Workgroup id -> (query block, head).  Consecutive ids go round-robin to the 8 XCDs, each with its
+// own L2, and every query block of a (b,h) reads that head's whole K and V: the blocks of one head
+// are therefore given consecutive slots of ONE XCD, so they run at the same time, walk the keys in
+// step and share each K/V tile through that L2 (with heads fastest, the heads resident on an XCD at
+// once need several times its L2 and most tiles come from memory again).  Longest block first
+// under a causal mask.
+__device__ __forceinline__ void prefill_block_to_tile(int block, int BH, int QB, bool longest_first, int &qb, int &bh)
+{
+    if (longest_first) { // query blocks in descending order across all heads
+        bh = block % BH;
+        qb = QB - 1 - block / BH;
+    } else if (BH % 8 == 0) {
+        const int x = block & 7, j = block >> 3;
+        bh = (j / QB) * 8 + x;
+        qb = QB - 1 - j % QB;
+    } else {
+        bh = block % BH;
+        qb = QB - 1 - block / BH;
+    }
+}
+
 // MFMA operand layouts used below (v_mfma_f32_32x32x2_f32, D += A(32x2) * B(2x32)):
 //   A: lane holds A[row = lane % 32][k = lane / 32];  B: lane holds B[k = lane / 32][col = lane % 32];
 //   D: register v of a lane holds D[row = 8*(v/4) + 4*(lane/32) + (v%4)][col = lane % 32].
@@ -130,7 +151,8 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
     __shared__ float sV[BN][LDK];
 
     const int BH = p.B * p.H;
-    const int qb = blockIdx.x / BH, bh = blockIdx.x % BH;
+    int qb, bh;
+    prefill_block_to_tile((int)blockIdx.x, BH, (p.S + kPrefillQueriesPerBlock - 1) / kPrefillQueriesPerBlock, false, qb, bh);
     const int S = p.S, P = p.start_pos, L = p.L;
     const int ctx = P + S;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -359,6 +381,8 @@ __device__ __forceinline__ float max16(const floatx16 &a)
 //
 // With a mask, tiles are processed according to their class (see above); tiles that every wave of
 // the workgroup skips are not even loaded.
+constexpr int kTileListCap = 1024; // tiles per pass over the context (32768 keys); longer contexts take several passes
+
 template <int D, bool HAS_MASK>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8)))
 void prefill_attn_f16_kernel(const PrefillParams p)
@@ -374,11 +398,12 @@ void prefill_attn_f16_kernel(const PrefillParams p)
 
     __shared__ __attribute__((aligned(16))) _Float16 sK[2][BN][LDK];
     __shared__ __attribute__((aligned(16))) _Float16 sV[2][BN][LDV];
-    __shared__ __attribute__((aligned(16))) float sM[HAS_MASK ? kPrefillQueriesPerBlock : 1][kMaskTileLd];
-    __shared__ int s_end;
+    __shared__ uint32_t s_list[HAS_MASK ? kTileListCap : 1];
+    __shared__ int s_wave_cnt[4];
 
     const int BH = p.B * p.H;
-    const int qb = blockIdx.x / BH, bh = blockIdx.x % BH;
+    int qb, bh;
+    prefill_block_to_tile((int)blockIdx.x, BH, (p.S + kPrefillQueriesPerBlock - 1) / kPrefillQueriesPerBlock, HAS_MASK, qb, bh);
     const int S = p.S, P = p.start_pos, L = p.L;
     const int ctx = P + S;
     const int NT = (ctx + BN - 1) / BN;
@@ -387,24 +412,34 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     const int q_row = qb * kPrefillQueriesPerBlock + wave * 32 + qi;
     const bool q_ok = q_row < S;
 
-    // last tile any wave of this workgroup needs
-    const uint32_t *cls = HAS_MASK ? p.tile_class + (size_t)qb * NT : nullptr;
-    int t_end = NT;
-    if constexpr (HAS_MASK) {
-        if (tid == 0) s_end = 0;
-        __syncthreads();
-        int last = 0;
-        for (int t = tid; t < NT; t += 256)
-            if (cls[t] != 0u) last = t + 1;
-        if (last > 0) atomicMax(&s_end, last);
-        __syncthreads();
-        t_end = s_end;
-    }
-    auto next_tile = [&](int t) { // uniform: the next tile some wave needs, or t_end
-        ++t;
-        if constexpr (HAS_MASK)
-            while (t < t_end && cls[t] == 0u) ++t;
-        return t;
+    // The tiles of [c0, c1) that some wave of this workgroup needs, in order, as a list in LDS:
+    // entry = tile << 8 | the four waves' classes (2 bits each).  Built once per chunk of
+    // kTileListCap tiles, so the loop below never chases a class word through memory.
+    auto build_list = [&](int c0, int c1) -> int {
+        int count = 0;
+        for (int base = c0; base < c1; base += 256) {
+            const int t = base + tid;
+            uint32_t w = 0;
+            if (t < c1) w = p.tile_class[(size_t)qb * NT + t];
+            const bool active = w != 0u;
+            const unsigned long long bal = __ballot(active);
+            if (lane == 0) s_wave_cnt[wave] = __popcll(bal);
+            __syncthreads();
+            int off = count;
+            for (int k = 0; k < wave; ++k) off += s_wave_cnt[k];
+            if (active) {
+                const uint32_t packed = (w & 3u) | ((w >> 8) & 3u) << 2 | ((w >> 16) & 3u) << 4 | ((w >> 24) & 3u) << 6;
+                s_list[off + __popcll(bal & ((1ull << lane) - 1ull))] = (uint32_t)t << 8 | packed;
+            }
+            count += s_wave_cnt[0] + s_wave_cnt[1] + s_wave_cnt[2] + s_wave_cnt[3];
+            __syncthreads();
+        }
+        return count;
+    };
+    // entry i of the current chunk; without a mask every tile is needed and every class is ZERO
+    auto list_entry = [&](int c0, int i) -> uint32_t {
+        if constexpr (HAS_MASK) return s_list[i];
+        else return (uint32_t)(c0 + i) << 8 | 0x55u;
     };
 
     half8 qreg[NC];
@@ -467,70 +502,80 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     // per-lane source of the transposing V reads: row 4hf + (lane%16)/4, halfs 16*((lane/16)%2) + 4*(lane%4)
     const int vrow = 4 * hf + ((lane & 15) >> 2), vcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
     const float inv_scale = 1.0f / p.scale;
+    const bool mask_vec4 = HAS_MASK && (p.mask_ld & 3) == 0 && (reinterpret_cast<uintptr_t>(p.attn_mask) & 15u) == 0;
 
     // The rotated queries must have landed before the loop: a wait inside it would also wait for
     // the tile prefetches that are meant to stay in flight.
 #pragma unroll
     for (int c = 0; c < NC; ++c) asm volatile("" : "+v"(qreg[c]));
 
-    // Software pipeline over the tiles this workgroup needs: tile t in LDS buffer `buf`, tile t1 in
-    // registers, the loads of tile t2 issued before tile t is multiplied.
-    int t = next_tile(-1);
-    if (t < t_end) {
-        fetch(t);
+    // Software pipeline over the listed tiles: entry e0's tile in LDS buffer `buf`, e1's in
+    // registers, the loads of e2's issued before e0's is multiplied; the list is read three entries
+    // ahead so that its LDS latency never stalls the loop.
+    for (int c0 = 0; c0 < NT; c0 += kTileListCap) {
+        const int c1 = min(c0 + kTileListCap, NT);
+        int n = c1 - c0;
+        if constexpr (HAS_MASK) n = build_list(c0, c1); // ends with a barrier: the tile buffers are free again
+        else if (c0 > 0) __syncthreads();
+        if (n == 0) continue;
+        uint32_t e0 = __builtin_amdgcn_readfirstlane(list_entry(c0, 0));
+        uint32_t e1 = n > 1 ? __builtin_amdgcn_readfirstlane(list_entry(c0, 1)) : 0u;
+        uint32_t e2 = n > 2 ? __builtin_amdgcn_readfirstlane(list_entry(c0, 2)) : 0u;
+        uint32_t e3 = n > 3 ? list_entry(c0, 3) : 0u;
+        fetch((int)(e0 >> 8));
         commit(0);
-        int t1 = next_tile(t);
-        if (t1 < t_end) fetch(t1);
+        if (n > 1) fetch((int)(e1 >> 8));
         int buf = 0;
-        while (true) {
+        for (int i = 0; i < n; ++i) {
+            const int t = (int)(e0 >> 8);
             __syncthreads(); // tile t is visible; every wave is done with the other buffer
-            int t2 = t_end;
-            if (t1 < t_end) {
-                commit(buf ^ 1);
-                t2 = next_tile(t1);
-                if (t2 < t_end) fetch(t2);
-            }
 
+            // The additive term enters as the initial value of the score accumulator, in units of the
+            // raw product: (s + mask/scale)*scale.  Zero for most tiles; the mask entries where the tile
+            // is mixed; -inf for keys beyond the context.  The mask is read before the prefetch below is
+            // issued: loads return in order, so waiting for it then does not wait for the prefetch.
             const int k0 = t * BN;
             uint32_t tc = kTileZero;
-            if constexpr (HAS_MASK) tc = __builtin_amdgcn_readfirstlane((cls[t] >> (8 * wave)) & 0xffu);
-            if (tc != kTileSkip) {
-                // The additive term enters as the initial value of the score accumulator, in units of
-                // the raw product: (s + mask/scale)*scale.  Zero for most tiles; the mask tile where it
-                // is mixed; -inf for keys beyond the context.
-                floatx16 st;
-                const half8 ka0 = *reinterpret_cast<const half8 *>(&sK[buf][qi][8 * hf]);
-                if (k0 + BN > ctx || tc == kTileMixed) {
+            if constexpr (HAS_MASK) tc = __builtin_amdgcn_readfirstlane((e0 >> (2 * wave)) & 3u);
+            const bool special = tc != kTileSkip && (k0 + BN > ctx || tc == kTileMixed);
+            floatx16 st;
+            if (special) {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) st[v] = 0.f;
-                    if constexpr (HAS_MASK) {
-                        if (tc == kTileMixed) {
-                            // this wave's 32 mask rows, coalesced (32 lanes read one 128-byte row segment), then
-                            // through the wave's own LDS rows into the score layout
-                            const int col = min(k0 + qi, ctx - 1);
-                            float mraw[16];
-#pragma unroll
-                            for (int j = 0; j < 16; ++j) {
-                                const int q = min(qb * kPrefillQueriesPerBlock + wave * 32 + 2 * j + hf, S - 1);
-                                mraw[j] = p.attn_mask[(size_t)(P + q) * p.mask_ld + col];
-                            }
-#pragma unroll
-                            for (int j = 0; j < 16; ++j) sM[wave * 32 + 2 * j + hf][qi] = mraw[j] * inv_scale;
-                            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                            __builtin_amdgcn_wave_barrier();
-                            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                for (int v = 0; v < 16; ++v) st[v] = 0.f;
+                if constexpr (HAS_MASK) {
+                    if (tc == kTileMixed) {
+                        // Mask entries of this lane's query, straight into the score layout (four runs of
+                        // four keys).  Only tiles that straddle a mask boundary come here — the diagonal
+                        // band of a causal mask — so the gather's poor coalescing does not matter; the
+                        // entries of keys beyond the context are overwritten below.
+                        const float *mrow = p.attn_mask + (size_t)(P + min(q_row, S - 1)) * p.mask_ld;
+                        if (mask_vec4 && k0 + BN <= ctx) {
 #pragma unroll
                             for (int g4 = 0; g4 < 4; ++g4) {
-                                const float4 x = *reinterpret_cast<const float4 *>(&sM[wave * 32 + qi][8 * g4 + 4 * hf]);
+                                const float4 x = *reinterpret_cast<const float4 *>(mrow + k0 + 8 * g4 + 4 * hf);
                                 st[4 * g4 + 0] = x.x; st[4 * g4 + 1] = x.y; st[4 * g4 + 2] = x.z; st[4 * g4 + 3] = x.w;
                             }
-                            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                            __builtin_amdgcn_wave_barrier(); // the rows are rewritten by this wave's next mixed tile
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) st[v] = mrow[min(k0 + 8 * (v / 4) + 4 * hf + (v % 4), ctx - 1)];
                         }
                     }
+                }
+            }
+
+            if (i + 1 < n) {
+                commit(buf ^ 1);
+                if (i + 2 < n) fetch((int)(e2 >> 8));
+            }
+
+            if (tc != kTileSkip) {
+                const half8 ka0 = *reinterpret_cast<const half8 *>(&sK[buf][qi][8 * hf]);
+                if (special) {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v)
+                    for (int v = 0; v < 16; ++v) {
+                        st[v] *= inv_scale;
                         if (k0 + 8 * (v / 4) + 4 * hf + (v % 4) >= ctx) st[v] = -__builtin_inff();
+                    }
                     st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka0, qreg[0], st, 0, 0, 0);
                 } else {
                     floatx16 zero;
@@ -586,25 +631,30 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                     }
             }
 
-            if (t1 >= t_end) break;
-            t = t1;
-            t1 = t2;
+            e0 = e1;
+            e1 = e2;
+            e2 = __builtin_amdgcn_readfirstlane(e3);
+            e3 = i + 4 < n ? list_entry(c0, i + 4) : 0u;
             buf ^= 1;
         }
     }
 
     l += __shfl_xor(l, 32);
     if (q_ok) {
+        // p = e / sum (decoder_kernels.cu:833) as one reciprocal and 64 products per lane: the quotient
+        // differs from a true division by an ulp, far inside the fp16 path's tolerance; a fully
+        // masked row still gives 0 * inf = NaN.
+        const float rl = 1.0f / l;
         float *dst = p.out + ((size_t)bh * S + q_row) * D;
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 float4 r;
-                r.x = ot[dt][4 * g4 + 0] / l;
-                r.y = ot[dt][4 * g4 + 1] / l;
-                r.z = ot[dt][4 * g4 + 2] / l;
-                r.w = ot[dt][4 * g4 + 3] / l;
+                r.x = ot[dt][4 * g4 + 0] * rl;
+                r.y = ot[dt][4 * g4 + 1] * rl;
+                r.z = ot[dt][4 * g4 + 2] * rl;
+                r.w = ot[dt][4 * g4 + 3] * rl;
                 *reinterpret_cast<float4 *>(dst + 32 * dt + 8 * g4 + 4 * hf) = r;
             }
     }

@@ -72,6 +72,79 @@ def test_prefill_strict_mask_first_row_is_nan(gpu):
     assert_out_close(out[:, :, 1:], want[:, :, 1:], "f32", "strict mask rows 1..")
 
 
+FMAX = float(np.finfo(np.float32).max)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+@pytest.mark.parametrize("S,P", [(300, 0), (257, 77), (128, 384), (40, 0)])
+def test_prefill_causal_mask_with_flt_max(gpu, dtype, S, P):
+    """The reference driver's mask value (samples/llama_fp16.cu:73-81): fully masked tiles contribute exact zeros
+    whether a kernel evaluates or drops them."""
+    L = 512
+    out, want, _ = run_both(gpu, 2, 3, 128, L, S, P, dtype, mask=causal_mask(L, -FMAX), seed=3 * S + P)
+    assert_out_close(out, want, dtype, f"-FLT_MAX causal S={S} P={P}")
+
+
+def test_prefill_strict_mask_first_row_is_nan_f16(gpu):
+    L = 192
+    m = np.where(np.arange(L)[:, None] > np.arange(L)[None, :], 0.0, -FMAX).astype(np.float32)
+    out, want, _ = run_both(gpu, 1, 2, 128, L, 150, 0, "f16", mask=m)
+    assert np.isnan(want[:, :, 0]).all() and np.isnan(out[:, :, 0]).all()
+    assert not np.isnan(out[:, :, 1:]).any()
+    assert_out_close(out[:, :, 1:], want[:, :, 1:], "f16", "strict mask rows 1.. (f16)")
+
+
+@pytest.mark.parametrize("fill", [-FMAX, -np.inf, -1e5])
+def test_prefill_sliding_window_mask_f16(gpu, fill):
+    """A band mask leaves fully masked tiles on both sides of the band: the kernel's tile list has gaps."""
+    L, S, P, win = 640, 200, 400, 96
+    i, j = np.arange(L)[:, None], np.arange(L)[None, :]
+    m = np.where((j > i) | (j < i - win), fill, 0.0).astype(np.float32)
+    out, want, _ = run_both(gpu, 2, 2, 128, L, S, P, "f16", mask=m, seed=5)
+    assert_out_close(out, want, "f16", f"sliding window fill={fill}")
+
+
+def test_prefill_dense_random_mask_f16(gpu):
+    """Every tile mixed: the general path, with a row stride that is not a multiple of four."""
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    B, H, D, L, S, P = 1, 3, 64, 200, 150, 30
+    ld = L + 3
+    rng = np.random.default_rng(7)
+    full = (rng.standard_normal((L, ld)) * 2).astype(np.float32)
+    full[rng.random((L, ld)) < 0.2] = -FMAX
+    full[:, 0] = 0.0  # no fully masked row
+    q, k, v, kc, vc, f = make(B, H, D, L, S, "f16", 9)
+    kc_ref, vc_ref = kc.copy(), vc.copy()
+    want = ref.prefill_attn(q, k, v, kc_ref, vc_ref, f, start_pos=P, attn_mask=np.ascontiguousarray(full[:, :L]),
+                            acc_double=True, threads=8)
+    t = lambda a: torch.from_numpy(a).to(gpu)
+    op = PrefillAttention(B, H, D, L, S, torch.float16, device=gpu)
+    out = op.prefill(t(q), t(k), t(v), t(kc), t(vc), t(f), start_pos=P, attn_mask=t(full), mask_ld=ld)
+    assert_out_close(out.cpu().numpy(), want, "f16", "dense random mask")
+
+
+def test_prefill_context_longer_than_one_tile_list_f16(gpu):
+    """More key tiles than one pass of the kernel's tile list holds (1024 tiles = 32768 keys).  The mask is a
+    single row shared by all queries (row stride 0): a key-padding mask that hides two long runs of keys."""
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    B, H, D, L, S = 1, 1, 32, 33100, 96
+    P = L - S
+    row = np.zeros(L, np.float32)
+    row[64:20000] = -FMAX
+    row[20040:32800] = -FMAX
+    q, k, v, kc, vc, f = make(B, H, D, L, S, "f16", 21)
+    t = lambda a: torch.from_numpy(a).to(gpu)
+    op = PrefillAttention(B, H, D, L, S, torch.float16, device=gpu)
+    for mask in (row, None):
+        want = ref.prefill_attn(q, k, v, kc.copy(), vc.copy(), f, start_pos=P, attn_mask=mask, mask_ld=0,
+                                acc_double=True, threads=8)
+        out = op.prefill(t(q), t(k), t(v), t(kc), t(vc), t(f), start_pos=P,
+                         attn_mask=None if mask is None else t(mask), mask_ld=0)
+        assert_out_close(out.cpu().numpy(), want, "f16", f"context of {L} keys, mask={'row' if mask is not None else None}")
+
+
 def test_prefill_literal_rope_rows(gpu):
     # reference as written: token s of the prompt is rotated by table row s (decoder_kernels.cu:440)
     out, want, _ = run_both(gpu, 2, 4, 128, 128, 60, 20, "f32", mask=causal_mask(128), rope_row=0)
