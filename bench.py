@@ -108,10 +108,10 @@ def bench_prefill(args) -> int:
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
     dense_flops = 4.0 * B * H * S * (P + S) * D  # every query against every key
-    # FLOPs the kernels execute: the fp16 kernel drops 32x32 tiles whose mask entries are all <= -1e30 (their
-    # weights are exactly 0); everything else, and the FP32 kernel always, multiplies every tile.
+    # FLOPs the kernels execute: 32x32 tiles whose mask entries are all <= -1e30 are dropped (their weights
+    # are exactly 0); every other tile is multiplied.
     flops = dense_flops
-    if w["dtype"] == "f16" and args.prefill_mask != "none":
+    if args.prefill_mask != "none":
         rows = mask_h[P:P + S, :P + S]
         pad_q, pad_k = (-S) % 32, (-(P + S)) % 32
         tiles = np.pad(rows, ((0, pad_q), (0, pad_k)), constant_values=-np.inf)

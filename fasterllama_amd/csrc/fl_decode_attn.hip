@@ -270,15 +270,16 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
     if (e != hipSuccess) return e;
     const unsigned qblocks = (unsigned)((p.S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock);
     const dim3 grid(qblocks * (unsigned)(p.B * p.H)); // mapped to (query block, head) by prefill_block_to_tile
+    if (p.attn_mask) {
+        const int ktiles = (p.start_pos + p.S + flattn::kPrefillKeysPerStep - 1) / flattn::kPrefillKeysPerStep;
+        hipLaunchKernelGGL(flattn::prefill_mask_classify_kernel, dim3((unsigned)ktiles, qblocks), dim3(256), 0, stream, p, ktiles);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     if constexpr (std::is_same<T, _Float16>::value) {
-        if (p.attn_mask) {
-            const int ktiles = (p.start_pos + p.S + flattn::kPrefillKeysPerStep - 1) / flattn::kPrefillKeysPerStep;
-            hipLaunchKernelGGL(flattn::prefill_mask_classify_kernel, dim3((unsigned)ktiles, qblocks), dim3(256), 0, stream, p,
-                               ktiles);
-            e = hipGetLastError();
-            if (e != hipSuccess) return e;
+        if (p.attn_mask)
             hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, true>), grid, dim3(256), 0, stream, p);
-        } else
+        else
             hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, false>), grid, dim3(256), 0, stream, p);
     } else {
         if (p.attn_mask)

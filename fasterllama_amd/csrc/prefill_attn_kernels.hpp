@@ -104,7 +104,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kPrefillQueriesPerBlock = 128; // 4 waves x 32 queries
 constexpr int kPrefillKeysPerStep = 32;
-constexpr int kMaskTileLd = kPrefillKeysPerStep + 4; // padded: 128-bit reads of 8 consecutive rows hit 32 banks
+constexpr uint32_t kTileSkip = 0, kTileZero = 1, kTileMixed = 2; // mask tile classes, see prefill_mask_classify_kernel
 
 // Workgroup id -> (query block, head).  Consecutive ids go round-robin to the 8 XCDs, each with its
 // own L2, and every query block of a (b,h) reads that head's whole K and V: the blocks of one head
@@ -136,7 +136,8 @@ __device__ __forceinline__ void prefill_block_to_tile(int block, int BH, int QB,
 // The contraction index of the first product is enumerated as d = 8c + 4*(lane/32) + r
 // (c = chunk, r = 0..3) so that each lane fetches its K operand as one 128-bit LDS read.
 template <typename T, int D, bool HAS_MASK>
-__global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) // two workgroups per compute unit
+void prefill_attn_kernel(const PrefillParams p)
 {
     typedef typename Vec16<T>::type V;
     constexpr int VEC = Vec16<T>::N;
@@ -152,7 +153,7 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
 
     const int BH = p.B * p.H;
     int qb, bh;
-    prefill_block_to_tile((int)blockIdx.x, BH, (p.S + kPrefillQueriesPerBlock - 1) / kPrefillQueriesPerBlock, false, qb, bh);
+    prefill_block_to_tile((int)blockIdx.x, BH, (p.S + kPrefillQueriesPerBlock - 1) / kPrefillQueriesPerBlock, HAS_MASK, qb, bh);
     const int S = p.S, P = p.start_pos, L = p.L;
     const int ctx = P + S;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -182,7 +183,21 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
     const T *Vb = reinterpret_cast<const T *>(p.v_cache) + (size_t)bh * L * D;
     const float scale = p.scale;
 
+    // Mask tile classes (see prefill_mask_classify_kernel): a tile no wave of the workgroup needs is
+    // neither loaded nor multiplied, a wave skips the tiles it alone does not need, and the mask is
+    // only read where it is not all zero.  Each of these leaves every bit of the result as it is:
+    // the dropped terms are exp(v - max) == 0 and fma(s, scale, 0) == s*scale.
+    const uint32_t *cls = HAS_MASK ? p.tile_class + (size_t)qb * ((ctx + BN - 1) / BN) : nullptr;
+    uint32_t word_next = HAS_MASK ? cls[0] : 0u;
+
     for (int k0 = 0; k0 < ctx; k0 += BN) {
+        uint32_t tc = kTileZero;
+        if constexpr (HAS_MASK) {
+            const uint32_t word = __builtin_amdgcn_readfirstlane(word_next);
+            if (k0 + BN < ctx) word_next = cls[k0 / BN + 1]; // in flight during this tile
+            if (word == 0u) continue;
+            tc = (word >> (8 * wave)) & 0xffu;
+        }
         __syncthreads(); // every wave is done with the previous tile
         for (int idx = tid; idx < BN * CPR; idx += 256) {
             const int r = idx / CPR, cc = idx % CPR;
@@ -210,9 +225,10 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int key = k0 + 8 * (v / 4) + 4 * hf + (v % 4);
-            mk[v] = (HAS_MASK && key < ctx) ? mrow[key] : 0.f;
+            mk[v] = (HAS_MASK && tc == kTileMixed && key < ctx) ? mrow[key] : 0.f;
         }
         __syncthreads();
+        if (tc == kTileSkip) continue; // wave-uniform; the barriers above are this iteration's only ones
 
         // S^T tile: 32 keys x 32 queries, contraction over D
         floatx16 st;
@@ -293,7 +309,6 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
 //   ZERO   drops the mask term where all entries are +-0;
 //   MIXED  evaluates the general form.
 // One 32-bit word per (128-query block, key tile): byte w is the class of the block's w-th wave.
-constexpr uint32_t kTileSkip = 0, kTileZero = 1, kTileMixed = 2;
 constexpr float kMaskedBelow = -1e30f;
 constexpr float kLazyMax = 8.0f; // base-2 units
 
