@@ -237,11 +237,11 @@ hipError_t dispatch_split(int D, const Params &p, dim3 grid, hipStream_t stream)
 
 bool prefill_head_dim_ok(int D) { return D == 32 || D == 64 || D == 128; }
 
-// Workspace layout of the prompt phase: [rotated queries B*H*S*D] [float output B*H*S*D (used when the
-// caller asks for INT8 only)] [mask tile classes: one word per 128-query block and 32-key tile, sized
-// for a context that fills the cache], each 256-byte aligned.
+// Workspace layout of the prompt phase: [float output B*H*S*D (used when the caller asks for INT8
+// only)] [mask tile classes: one word per 128-query block and 32-key tile, sized for a context that
+// fills the cache], each 256-byte aligned.
 struct PrefillWorkspace {
-    size_t q_rot, tmp_out, tile_class, total;
+    size_t tmp_out, tile_class, total;
 };
 
 PrefillWorkspace prefill_workspace(const fl_attn_desc *d, int S)
@@ -250,10 +250,9 @@ PrefillWorkspace prefill_workspace(const fl_attn_desc *d, int S)
     const size_t qblocks = ((size_t)S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock;
     const size_t ktiles = ((size_t)d->total_len + flattn::kPrefillKeysPerStep - 1) / flattn::kPrefillKeysPerStep;
     PrefillWorkspace w;
-    w.q_rot = 0;
-    w.tmp_out = n;
-    w.tile_class = 2 * n;
-    w.total = w.tile_class + align_up(qblocks * ktiles * sizeof(uint32_t), 256);
+    w.tmp_out = 0;
+    w.tile_class = n;
+    w.total = n + align_up(qblocks * ktiles * sizeof(uint32_t), 256);
     return w;
 }
 
@@ -498,7 +497,6 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     p.q = io->q; p.k_new = io->k_new; p.v_new = io->v_new;
     p.k_cache = io->k_cache; p.v_cache = io->v_cache;
     p.freq_cis = io->freq_cis; p.attn_mask = io->attn_mask;
-    p.q_rot = ws + wl.q_rot;
     p.tile_class = reinterpret_cast<uint32_t *>(ws + wl.tile_class);
     p.out = io->out ? io->out : reinterpret_cast<float *>(ws + wl.tmp_out);
     p.inp_scale = io->qkv_inp_scale; p.wq_scale = io->q_weight_scale;

@@ -9,11 +9,13 @@
 // 1e-5 parity bar of the FP32 path.  fp16 caches: fp16 MFMA (v_mfma_f32_32x32x16_f16) with FP32
 // accumulation (prefill_attn_f16_kernel).
 //
-// Two kernels:
-//   prefill_rope_append_kernel  elementwise: RoPE(q) -> workspace [B,H,S,D], RoPE(k), v ->
-//                               cache rows start_pos + s (bit-identical to the decode step's rows)
-//   prefill_attn_kernel         flash-attention style: a workgroup owns 128 queries of one (b,h)
-//                               (32 per wave) and walks the keys 32 at a time through LDS.
+// Kernels:
+//   prefill_rope_append_kernel    elementwise: RoPE(k), v -> cache rows start_pos + s (bit-identical
+//                                 to the decode step's rows)
+//   prefill_mask_classify_kernel  classes of the 32x32 tiles of the additive mask (skip / zero / mixed)
+//   prefill_attn_kernel,          flash-attention style: a workgroup owns 128 queries of one (b,h)
+//   prefill_attn_f16_kernel       (32 per wave), rotates them as it loads them, and walks the keys
+//                                 32 at a time through LDS.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -28,7 +30,6 @@ struct PrefillParams {
     void *k_cache, *v_cache;       // [B,H,L,D]
     const float *freq_cis;
     const float *attn_mask;
-    void *q_rot;  // workspace [B,H,S,D]: fp32 for FP32 caches, fp16 (the MFMA operand type) for fp16 caches
     uint32_t *tile_class; // workspace [ceil(S/128), ceil((start_pos+S)/32)]: mask tile classes (fp16 caches with a mask)
     float *out;   // [B,H,S,D] fp32
     const float *inp_scale, *wq_scale, *wk_scale, *wv_scale;
@@ -65,25 +66,19 @@ __global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillP
     const float inp_scale = is_i32 ? p.inp_scale[bs] : 0.f;
     const size_t in_off = (size_t)row * D;
     const size_t bh = (size_t)b * p.H + h;
-    T *qdst = reinterpret_cast<T *>(p.q_rot) + (bh * p.S + s) * D;
     T *kdst = reinterpret_cast<T *>(p.k_cache) + (bh * p.L + pos) * D;
     T *vdst = reinterpret_cast<T *>(p.v_cache) + (bh * p.L + pos) * D;
 
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
         const int e0 = (c * LPR + lig) * VEC;
-        float qx[VEC], kx[VEC], vx[VEC];
-        load_token_chunk<T, VEC>(p.q, in_off + e0, is_i32, inp_scale, is_i32 ? p.wq_scale + h * D + e0 : nullptr, qx);
+        float kx[VEC], vx[VEC];
         load_token_chunk<T, VEC>(p.k_new, in_off + e0, is_i32, inp_scale, is_i32 ? p.wk_scale + h * D + e0 : nullptr, kx);
         load_token_chunk<T, VEC>(p.v_new, in_off + e0, is_i32, inp_scale, is_i32 ? p.wv_scale + h * D + e0 : nullptr, vx);
-        V kt, vt, qt;
+        V kt, vt;
 #pragma unroll
         for (int i = 0; i < VEC; i += 4) {
             const float4 f = *reinterpret_cast<const float4 *>(freq + e0 + i);
-            float4 qo;
-            rope_pair(qx[i], qx[i + 1], f.x, f.y, qo.x, qo.y);
-            rope_pair(qx[i + 2], qx[i + 3], f.z, f.w, qo.z, qo.w);
-            qt[i] = (T)qo.x; qt[i + 1] = (T)qo.y; qt[i + 2] = (T)qo.z; qt[i + 3] = (T)qo.w;
             float r0, r1, r2, r3;
             rope_pair(kx[i], kx[i + 1], f.x, f.y, r0, r1);
             rope_pair(kx[i + 2], kx[i + 3], f.z, f.w, r2, r3);
@@ -92,13 +87,32 @@ __global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillP
         }
 #pragma unroll
         for (int i = 0; i < VEC; ++i) vt[i] = to_storage<T>(vx[i]);
-        *reinterpret_cast<V *>(qdst + e0) = qt;
         *reinterpret_cast<V *>(kdst + e0) = kt;
         *reinterpret_cast<V *>(vdst + e0) = vt;
     }
 }
 
 // ---------------------------------------------------------------- dense attention on MFMA
+
+// RoPE(q) for N consecutive head dims d0.. of one prompt token, in FP32: the attention kernels
+// rotate their own queries while they load them (decoder_kernels.cu:449-458), so the rotated
+// queries never travel through memory.  `token` indexes [B,S], `row` is the table row.
+template <typename T, int N>
+__device__ __forceinline__ void rotated_query_chunk(const PrefillParams &p, int D, int64_t token, int h, int d0, int row,
+                                                    float (&out)[N])
+{
+    const bool is_i32 = p.inp_scale != nullptr;
+    float x[N];
+    load_token_chunk<T, N>(p.q, (size_t)(token * p.H + h) * D + d0, is_i32, is_i32 ? p.inp_scale[token] : 0.f,
+                           is_i32 ? p.wq_scale + h * D + d0 : nullptr, x);
+    const float *freq = p.freq_cis + (size_t)row * D + d0;
+#pragma unroll
+    for (int i = 0; i < N; i += 4) {
+        const float4 f = *reinterpret_cast<const float4 *>(freq + i);
+        rope_pair(x[i], x[i + 1], f.x, f.y, out[i], out[i + 1]);
+        rope_pair(x[i + 2], x[i + 3], f.z, f.w, out[i + 2], out[i + 3]);
+    }
+}
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
@@ -163,12 +177,13 @@ void prefill_attn_kernel(const PrefillParams p)
 
     float qreg[NC][4];
     {
-        static_assert(std::is_same<T, float>::value, "the FP32-MFMA kernel reads FP32 rotated queries");
-        const float *qsrc = reinterpret_cast<const float *>(p.q_rot) + ((size_t)bh * S + (q_ok ? q_row : 0)) * D + 4 * hf;
+        static_assert(std::is_same<T, float>::value, "the FP32-MFMA kernel works on FP32 caches");
+        const int64_t token = (int64_t)(bh / p.H) * S + (q_ok ? q_row : 0);
+        const int row = (p.rope_row < 0 ? P : p.rope_row) + (q_ok ? q_row : 0);
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
-            float4 t = q_ok ? *reinterpret_cast<const float4 *>(qsrc + 8 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
-            qreg[c][0] = t.x; qreg[c][1] = t.y; qreg[c][2] = t.z; qreg[c][3] = t.w;
+            rotated_query_chunk<T, 4>(p, D, token, bh % p.H, 8 * c + 4 * hf, row, qreg[c]);
+            if (!q_ok) qreg[c][0] = qreg[c][1] = qreg[c][2] = qreg[c][3] = 0.f;
         }
     }
 
@@ -459,12 +474,14 @@ void prefill_attn_f16_kernel(const PrefillParams p)
 
     half8 qreg[NC];
     {
-        const _Float16 *qsrc = reinterpret_cast<const _Float16 *>(p.q_rot) + ((size_t)bh * S + (q_ok ? q_row : 0)) * D + 8 * hf;
+        const int64_t token = (int64_t)(bh / p.H) * S + (q_ok ? q_row : 0);
+        const int row = (p.rope_row < 0 ? P : p.rope_row) + (q_ok ? q_row : 0);
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
+            float x[8];
+            rotated_query_chunk<_Float16, 8>(p, D, token, bh % p.H, 16 * c + 8 * hf, row, x);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) qreg[c][i] = (_Float16)0;
-            if (q_ok) qreg[c] = *reinterpret_cast<const half8 *>(qsrc + 16 * c);
+            for (int i = 0; i < 8; ++i) qreg[c][i] = q_ok ? (_Float16)x[i] : (_Float16)0; // rounded once, as an MFMA operand
         }
     }
 
