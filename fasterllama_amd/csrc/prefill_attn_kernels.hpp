@@ -426,8 +426,16 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     constexpr int LPT = (BN * CPR + 255) / 256; // chunks per thread per tile, for K and for V
     static_assert(D % 32 == 0, "head size must be a multiple of 32");
 
-    __shared__ __attribute__((aligned(16))) _Float16 sK[2][BN][LDK];
-    __shared__ __attribute__((aligned(16))) _Float16 sV[2][BN][LDV];
+    constexpr int LDQ = D + 8;              // halfs; the workgroup's rotated queries pass through the tile buffers once
+    constexpr int HALF_D = D >= 128 ? 64 : 32; // output columns per epilogue pass
+    constexpr int LDO = HALF_D + 4;         // floats; the output block passes through the tile buffers too
+    constexpr int TILE_HALFS = 2 * BN * (LDK + LDV), Q_HALFS = kPrefillQueriesPerBlock * LDQ,
+                  O_HALFS = kPrefillQueriesPerBlock * LDO * 2;
+    constexpr int SMEM_HALFS = TILE_HALFS > Q_HALFS ? (TILE_HALFS > O_HALFS ? TILE_HALFS : O_HALFS)
+                                                    : (Q_HALFS > O_HALFS ? Q_HALFS : O_HALFS);
+    __shared__ __attribute__((aligned(16))) _Float16 smem[SMEM_HALFS];
+    _Float16 (*sK)[BN][LDK] = reinterpret_cast<_Float16 (*)[BN][LDK]>(smem);
+    _Float16 (*sV)[BN][LDV] = reinterpret_cast<_Float16 (*)[BN][LDV]>(smem + 2 * BN * LDK);
     __shared__ uint32_t s_list[HAS_MASK ? kTileListCap : 1];
     __shared__ int s_wave_cnt[4];
 
@@ -440,7 +448,6 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int qi = lane & 31, hf = lane >> 5;
     const int q_row = qb * kPrefillQueriesPerBlock + wave * 32 + qi;
-    const bool q_ok = q_row < S;
 
     // The tiles of [c0, c1) that some wave of this workgroup needs, in order, as a list in LDS:
     // entry = tile << 8 | the four waves' classes (2 bits each).  Built once per chunk of
@@ -472,17 +479,33 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         else return (uint32_t)(c0 + i) << 8 | 0x55u;
     };
 
+    // Rotated queries of the workgroup: loaded and rotated cooperatively (16 lanes per 256-byte row, so
+    // the [B,S,H,D] rows are read whole), rounded once to fp16 as MFMA operands, and handed to their
+    // lanes through LDS.  Reading them per lane instead — 32 rows a wave, 16 bytes a lane — keeps the
+    // texture units busy for longer than ten key tiles take.
     half8 qreg[NC];
     {
-        const int64_t token = (int64_t)(bh / p.H) * S + (q_ok ? q_row : 0);
-        const int row = (p.rope_row < 0 ? P : p.rope_row) + (q_ok ? q_row : 0);
+        const int b = bh / p.H, h = bh % p.H;
+        const int row0 = p.rope_row < 0 ? P : p.rope_row;
+        for (int idx = tid; idx < kPrefillQueriesPerBlock * CPR; idx += 256) {
+            const int r = idx / CPR, cc = idx % CPR;
+            const int q = qb * kPrefillQueriesPerBlock + r;
+            half8 hq;
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            float x[8];
-            rotated_query_chunk<_Float16, 8>(p, D, token, bh % p.H, 16 * c + 8 * hf, row, x);
+            for (int i = 0; i < 8; ++i) hq[i] = (_Float16)0;
+            if (q < S) {
+                float x[8];
+                rotated_query_chunk<_Float16, 8>(p, D, (int64_t)b * S + q, h, cc * 8, row0 + q, x);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) qreg[c][i] = q_ok ? (_Float16)x[i] : (_Float16)0; // rounded once, as an MFMA operand
+                for (int i = 0; i < 8; ++i) hq[i] = (_Float16)x[i];
+            }
+            *reinterpret_cast<half8 *>(smem + r * LDQ + cc * 8) = hq;
         }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+            qreg[c] = *reinterpret_cast<const half8 *>(smem + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
+        __syncthreads(); // the tile buffers are free for K and V
     }
 
     floatx16 ot[NDT];
@@ -671,24 +694,43 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         }
     }
 
+    // Epilogue: p = e / sum (decoder_kernels.cu:833) as one reciprocal and 64 products per lane (the
+    // quotient differs from a true division by an ulp, far inside the fp16 path's tolerance; a fully
+    // masked row still gives 0 * inf = NaN).  The lane's values are 16-byte pieces of 32 different
+    // output rows; each wave turns its 32 x D block through its own slice of the tile buffers so that
+    // the global stores are whole 256-byte row segments.
     l += __shfl_xor(l, 32);
-    if (q_ok) {
-        // p = e / sum (decoder_kernels.cu:833) as one reciprocal and 64 products per lane: the quotient
-        // differs from a true division by an ulp, far inside the fp16 path's tolerance; a fully
-        // masked row still gives 0 * inf = NaN.
-        const float rl = 1.0f / l;
-        float *dst = p.out + ((size_t)bh * S + q_row) * D;
+    const float rl = 1.0f / l;
+    __syncthreads(); // every wave is done with the last K/V tile
+    {
+        float *so = reinterpret_cast<float *>(smem) + wave * 32 * LDO;
+        const int q0 = qb * kPrefillQueriesPerBlock + wave * 32;
+        float *dst0 = p.out + ((size_t)bh * S + q0) * D;
+        constexpr int LPRW = HALF_D / 4;               // lanes per row when reading back
+        constexpr int RPI = 64 / LPRW;                 // rows per store instruction
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
+        for (int pass = 0; pass < D / HALF_D; ++pass) {
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                float4 r;
-                r.x = ot[dt][4 * g4 + 0] * rl;
-                r.y = ot[dt][4 * g4 + 1] * rl;
-                r.z = ot[dt][4 * g4 + 2] * rl;
-                r.w = ot[dt][4 * g4 + 3] * rl;
-                *reinterpret_cast<float4 *>(dst + 32 * dt + 8 * g4 + 4 * hf) = r;
+            for (int dd = 0; dd < HALF_D / 32; ++dd) {
+                const int dt = pass * (HALF_D / 32) + dd;
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4)
+                    *reinterpret_cast<float4 *>(so + qi * LDO + 32 * dd + 8 * g4 + 4 * hf) =
+                        make_float4(ot[dt][4 * g4 + 0] * rl, ot[dt][4 * g4 + 1] * rl, ot[dt][4 * g4 + 2] * rl,
+                                    ot[dt][4 * g4 + 3] * rl);
             }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int r0 = 0; r0 < 32; r0 += RPI) {
+                const int r = r0 + lane / LPRW, c4 = lane % LPRW;
+                const float4 v = *reinterpret_cast<const float4 *>(so + r * LDO + 4 * c4);
+                if (q0 + r < S) *reinterpret_cast<float4 *>(dst0 + (size_t)r * D + pass * HALF_D + 4 * c4) = v;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier(); // the slice is rewritten by the next pass
+        }
     }
 }
 
