@@ -316,13 +316,13 @@ void prefill_attn_kernel(const PrefillParams p)
 // The additive mask is caller data, but the masks that occur in practice are piecewise trivial: a
 // causal mask is all zero below the diagonal band and all "minus huge" above it.  A small kernel
 // classifies every 32-query x 32-key tile of the mask rows this call uses, once per call (the mask
-// is shared by all (b,h)), and the fp16 attention kernel then
-//   SKIP   never touches a tile whose entries are all <= -1e30: with finite K the scores
+// is shared by all (b,h)), and the attention kernels then
+//   SKIP   never touch a tile whose entries are all <= -1e30: with finite K the scores
 //          v = s*scale + mask stay below every running maximum (floor -1e9) and exp(v - max) is
 //          exactly 0, so the tile contributes exact zeros to the sum and the output — skipping it
 //          is bit-identical to evaluating it (decoder_kernels.cu:811-833 arithmetic);
-//   ZERO   drops the mask term where all entries are +-0;
-//   MIXED  evaluates the general form.
+//   ZERO   drop the mask term where all entries are +-0 (fma(s, scale, 0) == s*scale);
+//   MIXED  evaluate the general form.
 // One 32-bit word per (128-query block, key tile): byte w is the class of the block's w-th wave.
 constexpr float kMaskedBelow = -1e30f;
 constexpr float kLazyMax = 8.0f; // base-2 units
@@ -400,6 +400,8 @@ __device__ __forceinline__ float max16(const floatx16 &a)
 // MFMAs).  Per score the common tile costs: 1/2 v_max3 (maximum over the raw products; the scale is
 // positive, so it commutes with max), 1 v_fma (s*scale - m), 1 v_exp, 1/2 v_cvt_pk_f16_f32 and
 // 1/2 v_dot2c_f32_f16 (the row sum, taken over the rounded probabilities that are multiplied in).
+// The additive mask and the -inf of keys past the context enter as the initial value of the score
+// accumulator; the output accumulators are rescaled lazily (kLazyMax).
 //
 // Data path: K and V tiles (32 keys) are double-buffered in LDS, row-major with padded rows; loads of
 // tile t+2 are in flight in registers while tile t is multiplied, one barrier per tile.  The first
@@ -409,8 +411,8 @@ __device__ __forceinline__ float max16(const floatx16 &a)
 // 0..3), so V is never transposed in memory.  Contraction slots of the second product: a lane-half
 // hf holds the keys 16u + 4hf + r (r < 4) and 16u + 8 + 4hf + (r - 4) after the first.
 //
-// With a mask, tiles are processed according to their class (see above); tiles that every wave of
-// the workgroup skips are not even loaded.
+// With a mask, tiles are processed according to their class (see above): each workgroup compacts the
+// tiles some wave of it needs into a list in LDS, and tiles that every wave skips are not even loaded.
 constexpr int kTileListCap = 1024; // tiles per pass over the context (32768 keys); longer contexts take several passes
 
 template <int D, bool HAS_MASK>
