@@ -184,6 +184,8 @@ def main() -> int:
                     help="'all' prints one JSON line per configuration cfg1..cfg5 (each in a child process)")
     ap.add_argument("--nsplit", type=int, default=0, help="force the context split count (0 = library's choice)")
     ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--graph-steps", type=int, default=20,
+                    help="also time the step replayed from a HIP graph of this many steps (0 = skip)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="only run a plain 1 GiB -> 1 GiB elementwise copy kernel a few times (for scaling "
@@ -327,6 +329,35 @@ def main() -> int:
     torch.cuda.synchronize()
     kern_ms = ev2.elapsed_time(ev3) / args.steps
 
+    # ---- the same step replayed from a HIP graph (how a serving loop hides launch gaps): G steps per
+    # graph, rotating over the cache copies like the eager loop; reported beside the eager figure
+    graph_us = None
+    if args.graph_steps > 0:
+        G = max(copies, args.graph_steps // copies * copies)
+        side = torch.cuda.Stream(device=dev)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                cs = torch.cuda.current_stream(dev)
+                for i in range(G):
+                    st = op.launch(ios[i % copies], stream=cs)
+                    if st != 0:
+                        raise capi.FlAttnError(st, capi.strerror(st))
+        torch.cuda.synchronize()
+        reps = max(1, args.steps // G)
+        for _ in range(2):
+            g.replay()
+        torch.cuda.synchronize()
+        ev4, ev5 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev4.record(stream)
+        for _ in range(reps):
+            g.replay()
+        ev5.record(stream)
+        torch.cuda.synchronize()
+        graph_us = ev4.elapsed_time(ev5) / (reps * G) * 1e3
+        if not np.array_equal(out.cpu().numpy(), out_gpu):
+            raise RuntimeError("HIP-graph replay and eager step disagree")
+
     alg = algorithmic_bytes(B, H, D, e, sum_ctx)
     gbps = alg / (step_ms * 1e-3) / 1e9
     kern_gbps = alg / (kern_ms * 1e-3) / 1e9
@@ -400,6 +431,7 @@ def main() -> int:
             "kernel": "decode_attn_split_kernel", "kernel_us": round(kern_ms * 1e3, 2),
         },
         "cpu_baseline": cpu,
+        "hip_graph_us_per_step": None if graph_us is None else round(graph_us, 2),
         "host_ms_total": round(host_ms, 3),
         "input_gen_s": round(gen_s, 2),
     }
