@@ -85,6 +85,14 @@ def test_prefill_causal_mask_with_flt_max(gpu, dtype, S, P):
     assert_out_close(out, want, dtype, f"-FLT_MAX causal S={S} P={P}")
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+@pytest.mark.parametrize("D", [32, 64])
+def test_prefill_small_heads_with_causal_mask(gpu, dtype, D):
+    L = 320
+    out, want, _ = run_both(gpu, 2, 4, D, L, 200, 100, dtype, mask=causal_mask(L, -FMAX), seed=D + 1)
+    assert_out_close(out, want, dtype, f"D={D} -FLT_MAX causal")
+
+
 def test_prefill_strict_mask_first_row_is_nan_f16(gpu):
     L = 192
     m = np.where(np.arange(L)[:, None] > np.arange(L)[None, :], 0.0, -FMAX).astype(np.float32)
