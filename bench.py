@@ -88,7 +88,7 @@ def bench_prefill(args) -> int:
     kc = torch.zeros(B, H, L, D, dtype=t_dt, device=dev)
     vc = torch.zeros_like(kc)
     out = torch.empty(B, H, S, D, dtype=torch.float32, device=dev)
-    op = PrefillAttention(B, H, D, L, S, t_dt, device=dev)
+    op = PrefillAttention(B, H, D, L, S, t_dt, device=dev, fast_qk=args.prefill_fast_qk)
     io = op.make_io(q, k, v, kc, vc, freq, out, start_pos=P, attn_mask=None if args.prefill_mask == "none" else mask)
     stream = torch.cuda.current_stream(dev)
 
@@ -147,7 +147,8 @@ def bench_prefill(args) -> int:
                                + {"causal": "causal additive mask, -FLT_MAX above the diagonal",
                                   "causal-1e5": "causal additive mask, -1e5 above the diagonal",
                                   "block-causal": "additive mask, causal over blocks of 128 tokens, -FLT_MAX above",
-                                  "none": "no mask"}[args.prefill_mask],
+                                  "none": "no mask"}[args.prefill_mask]
+                               + (", fast first product (fp16 queries)" if args.prefill_fast_qk and w["dtype"] == "f16" else ""),
                    "flops_per_step": flops, "dense_flops_per_step": dense_flops,
                    "tokens_per_s": round(B * S / (ms * 1e-3), 1)},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": peak, "unit": "TFLOP/s",
@@ -194,6 +195,8 @@ def main() -> int:
     ap.add_argument("--prefill-mask", default="causal", choices=["causal", "causal-1e5", "block-causal", "none"],
                     help="prompt-phase workloads: additive causal mask with -FLT_MAX (the reference's driver) or "
                          "-1e5 (its kernel harness) above the diagonal, or no mask")
+    ap.add_argument("--prefill-fast-qk", action="store_true",
+                    help="prompt-phase fp16 workloads: FL_ATTN_FLAG_FAST_PROMPT_QK (queries as one fp16 value)")
     ap.add_argument("--segment", default="attention", choices=["attention", "int32-int8"],
                     help="attention: q/k/v in the cache dtype -> float output (the headline metric). "
                          "int32-int8: the whole reference segment, int32 GEMM accumulators + scales in, "

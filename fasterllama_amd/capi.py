@@ -15,6 +15,7 @@ LIB_PATH = os.environ.get("FL_DECODE_ATTN_LIB") or os.path.join(_PKG, "lib", "li
 FL_ATTN_F32 = 0
 FL_ATTN_F16 = 1
 FL_ATTN_ROPE_AT_POSITION = -1
+FL_ATTN_FLAG_FAST_PROMPT_QK = 1
 
 FL_ATTN_OK = 0
 FL_ATTN_ERR_NULL_POINTER = -1
@@ -52,7 +53,7 @@ class AttnDesc(C.Structure):
         ("dtype", C.c_int32),
         ("nsplit", C.c_int32),
         ("softmax_scale", C.c_float),
-        ("reserved", C.c_int32),
+        ("flags", C.c_int32),
     ]
 
 

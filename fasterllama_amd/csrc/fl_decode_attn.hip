@@ -65,7 +65,7 @@ int validate_desc(const fl_attn_desc *d)
     if (d->batch_size <= 0 || d->head_num <= 0 || d->total_len <= 0) return FL_ATTN_ERR_SHAPE;
     if (d->batch_size > 65535 || d->head_num > 65535) return FL_ATTN_ERR_SHAPE;
     if (!head_dim_ok(d->size_per_head)) return FL_ATTN_ERR_HEAD_DIM;
-    if (d->nsplit < 0 || d->nsplit > kMaxSplits || d->reserved != 0) return FL_ATTN_ERR_ARGUMENT;
+    if (d->nsplit < 0 || d->nsplit > kMaxSplits || (d->flags & ~FL_ATTN_FLAG_FAST_PROMPT_QK) != 0) return FL_ATTN_ERR_ARGUMENT;
     if (!(d->softmax_scale >= 0.f) || std::isinf(d->softmax_scale)) return FL_ATTN_ERR_ARGUMENT;
     // the streaming grid is one-dimensional: B*H*splits workgroups must fit the 2^31 limit
     if ((int64_t)d->batch_size * d->head_num > (int64_t)INT32_MAX / kMaxSplits) return FL_ATTN_ERR_SHAPE;
@@ -276,10 +276,14 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
         if (e != hipSuccess) return e;
     }
     if constexpr (std::is_same<T, _Float16>::value) {
-        if (p.attn_mask)
-            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, true>), grid, dim3(256), 0, stream, p);
+        if (p.attn_mask && p.fast_qk)
+            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, true, false>), grid, dim3(256), 0, stream, p);
+        else if (p.attn_mask)
+            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, true, true>), grid, dim3(256), 0, stream, p);
+        else if (p.fast_qk)
+            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, false, false>), grid, dim3(256), 0, stream, p);
         else
-            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, false>), grid, dim3(256), 0, stream, p);
+            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, false, true>), grid, dim3(256), 0, stream, p);
     } else {
         if (p.attn_mask)
             hipLaunchKernelGGL((flattn::prefill_attn_kernel<T, D, true>), grid, dim3(256), 0, stream, p);
@@ -505,6 +509,7 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     p.B = desc->batch_size; p.H = desc->head_num; p.L = L; p.S = seq_len;
     p.start_pos = io->start_pos; p.rope_row = io->rope_row;
     p.scale = desc->softmax_scale > 0.f ? desc->softmax_scale : 1.0f / sqrtf((float)D);
+    p.fast_qk = (desc->flags & FL_ATTN_FLAG_FAST_PROMPT_QK) != 0;
 
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     hipError_t e = desc->dtype == FL_ATTN_F16 ? dispatch_prefill<_Float16>(D, p, stream) : dispatch_prefill<float>(D, p, stream);

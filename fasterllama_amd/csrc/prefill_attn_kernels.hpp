@@ -37,6 +37,7 @@ struct PrefillParams {
     int32_t B, H, L, S;
     int32_t start_pos, rope_row;
     float scale;
+    int32_t fast_qk; // fp16 kernel: rotated queries as one fp16 value instead of an fp16 pair
 };
 
 // ---------------------------------------------------------------- RoPE + transpose + append
@@ -415,7 +416,7 @@ __device__ __forceinline__ float max16(const floatx16 &a)
 // tiles some wave of it needs into a list in LDS, and tiles that every wave skips are not even loaded.
 constexpr int kTileListCap = 1024; // tiles per pass over the context (32768 keys); longer contexts take several passes
 
-template <int D, bool HAS_MASK>
+template <int D, bool HAS_MASK, bool QSPLIT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8)))
 void prefill_attn_f16_kernel(const PrefillParams p)
 {
@@ -486,20 +487,29 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     // lanes through LDS.  Reading them per lane instead — 32 rows a wave, 16 bytes a lane — keeps the
     // texture units busy for longer than ten key tiles take.
     half8 qreg[NC];
+    half8 qlo[QSPLIT ? NC : 1]; // remainders q - fp16(q): the first product runs on the pair, see below
     {
         const int b = bh / p.H, h = bh % p.H;
         const int row0 = p.rope_row < 0 ? P : p.rope_row;
-        for (int idx = tid; idx < kPrefillQueriesPerBlock * CPR; idx += 256) {
+        constexpr int QPT = kPrefillQueriesPerBlock * CPR / 256; // 16-byte chunks per thread
+        half8 lo_keep[QSPLIT ? QPT : 1];
+#pragma unroll
+        for (int j = 0; j < QPT; ++j) {
+            const int idx = tid + j * 256;
             const int r = idx / CPR, cc = idx % CPR;
             const int q = qb * kPrefillQueriesPerBlock + r;
             half8 hq;
 #pragma unroll
             for (int i = 0; i < 8; ++i) hq[i] = (_Float16)0;
+            if constexpr (QSPLIT) lo_keep[j] = hq;
             if (q < S) {
                 float x[8];
                 rotated_query_chunk<_Float16, 8>(p, D, (int64_t)b * S + q, h, cc * 8, row0 + q, x);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) hq[i] = (_Float16)x[i];
+                for (int i = 0; i < 8; ++i) {
+                    hq[i] = (_Float16)x[i];
+                    if constexpr (QSPLIT) lo_keep[j][i] = (_Float16)(x[i] - (float)hq[i]);
+                }
             }
             *reinterpret_cast<half8 *>(smem + r * LDQ + cc * 8) = hq;
         }
@@ -507,7 +517,20 @@ void prefill_attn_f16_kernel(const PrefillParams p)
 #pragma unroll
         for (int c = 0; c < NC; ++c)
             qreg[c] = *reinterpret_cast<const half8 *>(smem + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
-        __syncthreads(); // the tile buffers are free for K and V
+        __syncthreads();
+        if constexpr (QSPLIT) {
+#pragma unroll
+            for (int j = 0; j < QPT; ++j) {
+                const int idx = tid + j * 256;
+                *reinterpret_cast<half8 *>(smem + (idx / CPR) * LDQ + (idx % CPR) * 8) = lo_keep[j];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+                qlo[c] = *reinterpret_cast<const half8 *>(smem + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
+            __syncthreads();
+        }
+        // the tile buffers are free for K and V
     }
 
     floatx16 ot[NDT];
@@ -640,10 +663,15 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                     for (int v = 0; v < 16; ++v) zero[v] = 0.f;
                     st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka0, qreg[0], zero, 0, 0, 0); // the literal 0 operand
                 }
+                // With QSPLIT every K operand multiplies the query's fp16 value and its remainder: the pair
+                // carries 22 significant bits, so the scores keep FP32-level accuracy at any magnitude
+                // (a single fp16 query leaves |s| * 2^-12 of error in each score).
+                if constexpr (QSPLIT) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka0, qlo[0], st, 0, 0, 0);
 #pragma unroll
                 for (int c = 1; c < NC; ++c) {
                     const half8 ka = *reinterpret_cast<const half8 *>(&sK[buf][qi][16 * c + 8 * hf]);
                     st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[c], st, 0, 0, 0);
+                    if constexpr (QSPLIT) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qlo[c], st, 0, 0, 0);
                 }
 
                 // Softmax update of this lane's query (decoder_kernels.cu:811-833 in base 2).  The reference

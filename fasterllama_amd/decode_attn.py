@@ -104,8 +104,10 @@ class PrefillAttention(DecodeAttention):
 
     def __init__(self, batch_size: int, head_num: int, size_per_head: int, total_len: int, max_seq_len: int,
                  dtype: torch.dtype = torch.float16, softmax_scale: float = 0.0,
-                 device: str | torch.device = "cuda:0"):
+                 device: str | torch.device = "cuda:0", fast_qk: bool = False):
         super().__init__(batch_size, head_num, size_per_head, total_len, dtype, 0, softmax_scale, device)
+        if fast_qk:  # fp16 caches: queries as one fp16 value in the first product (see FL_ATTN_FLAG_FAST_PROMPT_QK)
+            self.desc.flags |= capi.FL_ATTN_FLAG_FAST_PROMPT_QK
         n = C.c_size_t(0)
         capi.check(self.lib.fl_prefill_attn_workspace_bytes(C.byref(self.desc), max_seq_len, C.byref(n)))
         self.max_seq_len = max_seq_len

@@ -60,6 +60,13 @@ typedef enum fl_attn_status {
 
 enum { FL_ATTN_F32 = 0, FL_ATTN_F16 = 1 };
 
+/* fl_attn_desc.flags.
+ * FL_ATTN_FLAG_FAST_PROMPT_QK (prompt phase with FL_ATTN_F16 caches only): the rotated queries enter the
+ * matrix cores rounded once to fp16 instead of as an fp16 pair (value + remainder).  The first product
+ * costs half the MFMAs; each score s then carries an error of about |s| * 2^-12, harmless for scores
+ * of a few units and visible (1e-2 on the output) when keys are scaled so that |s| reaches 30-90. */
+#define FL_ATTN_FLAG_FAST_PROMPT_QK 1
+
 /* rope_row value meaning "rotate by the table row of each sequence's own position" */
 #define FL_ATTN_ROPE_AT_POSITION (-1)
 
@@ -72,7 +79,7 @@ typedef struct fl_attn_desc {
     int32_t dtype;         /* storage type of q/k_new/v_new and of both caches */
     int32_t nsplit;        /* context splits per (b,h); 0 = chosen by the library */
     float softmax_scale;   /* 0 = 1/sqrt(D) (open_decoder.cu:208) */
-    int32_t reserved;      /* must be 0 */
+    int32_t flags;         /* 0, or a combination of the FL_ATTN_FLAG_ values below */
 } fl_attn_desc;
 
 /* Per-call operands; mirrors the arguments of OpenDecoder::forward (open_decoder.h:76-77). */

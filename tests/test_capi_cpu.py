@@ -12,7 +12,7 @@ from fasterllama_amd import capi
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def desc(B=2, H=4, D=128, L=64, dtype=capi.FL_ATTN_F16, nsplit=0, scale=0.0, reserved=0):
+def desc(B=2, H=4, D=128, L=64, dtype=capi.FL_ATTN_F16, nsplit=0, scale=0.0, reserved=0):  # reserved: the flags word
     return capi.AttnDesc(B, H, D, L, dtype, nsplit, scale, reserved)
 
 
@@ -64,7 +64,8 @@ def test_strerror_covers_every_status():
     (dict(nsplit=5000), capi.FL_ATTN_ERR_ARGUMENT),
     (dict(scale=-1.0), capi.FL_ATTN_ERR_ARGUMENT),
     (dict(scale=float("nan")), capi.FL_ATTN_ERR_ARGUMENT),
-    (dict(reserved=1), capi.FL_ATTN_ERR_ARGUMENT),
+    (dict(reserved=2), capi.FL_ATTN_ERR_ARGUMENT),   # unknown flag bit
+    (dict(reserved=-1), capi.FL_ATTN_ERR_ARGUMENT),
 ])
 def test_descriptor_validation(kw, want):
     lib = capi.load()

@@ -93,6 +93,50 @@ def test_prefill_small_heads_with_causal_mask(gpu, dtype, D):
     assert_out_close(out, want, dtype, f"D={D} -FLT_MAX causal")
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_prefill_sharp_softmax_with_scaled_keys(gpu, dtype):
+    """Some key rows scaled by 8 (the stress of BASELINE configuration 4): near one-hot weights, running maxima
+    that jump late in the walk over the keys, and scores far above the lazily updated reference maximum."""
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    B, H, D, L, S = 1, 4, 128, 512, 400
+    q, k, v, kc, vc, f = make(B, H, D, L, S, dtype, 33)
+    for r in (5, 130, 131, 399):
+        k[:, r] *= 8
+    q[:, 200:] *= 3
+    mask = causal_mask(L, -FMAX)
+    kc_ref, vc_ref = kc.copy(), vc.copy()
+    want = ref.prefill_attn(q, k, v, kc_ref, vc_ref, f, attn_mask=mask, acc_double=True, threads=8)
+    t = lambda a: torch.from_numpy(a).to(gpu)
+    op = PrefillAttention(B, H, D, L, S, torch.float16 if dtype == "f16" else torch.float32, device=gpu)
+    out = op.prefill(t(q), t(k), t(v), t(kc), t(vc), t(f), attn_mask=t(mask)).cpu().numpy()
+    assert np.isfinite(out).all()
+    assert_out_close(out, want, dtype, "scaled keys")
+    if dtype == "f16":
+        # the opt-in fast first product rounds the rotated queries to fp16: scores of magnitude ~90 then
+        # carry ~2e-2 of error each, which this data makes visible (and ordinary data does not)
+        fast = PrefillAttention(B, H, D, L, S, torch.float16, device=gpu, fast_qk=True)
+        out_fast = fast.prefill(t(q), t(k), t(v), t(kc), t(vc), t(f), attn_mask=t(mask)).cpu().numpy()
+        err = np.abs(out_fast - want).max()
+        assert 2e-3 < err < 5e-2, err
+
+
+def test_prefill_fast_qk_meets_the_bar_on_ordinary_data(gpu):
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    B, H, D, L, S, P = 2, 3, 128, 512, 300, 60
+    q, k, v, kc, vc, f = make(B, H, D, L, S, "f16", 5)
+    mask = causal_mask(L, -FMAX)
+    want = ref.prefill_attn(q, k, v, kc.copy(), vc.copy(), f, start_pos=P, attn_mask=mask, acc_double=True, threads=8)
+    t = lambda a: torch.from_numpy(a).to(gpu)
+    for msk in (mask, None):
+        if msk is None:
+            want = ref.prefill_attn(q, k, v, kc.copy(), vc.copy(), f, start_pos=P, acc_double=True, threads=8)
+        op = PrefillAttention(B, H, D, L, S, torch.float16, device=gpu, fast_qk=True)
+        out = op.prefill(t(q), t(k), t(v), t(kc), t(vc), t(f), start_pos=P, attn_mask=None if msk is None else t(msk))
+        assert_out_close(out.cpu().numpy(), want, "f16", "fast first product")
+
+
 def test_prefill_strict_mask_first_row_is_nan_f16(gpu):
     L = 192
     m = np.where(np.arange(L)[:, None] > np.arange(L)[None, :], 0.0, -FMAX).astype(np.float32)
