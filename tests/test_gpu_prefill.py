@@ -197,6 +197,36 @@ def test_prefill_context_longer_than_one_tile_list_f16(gpu):
         assert_out_close(out.cpu().numpy(), want, "f16", f"context of {L} keys, mask={'row' if mask is not None else None}")
 
 
+def test_prefill_hip_graph_replay_matches_eager(gpu):
+    """The prompt-phase call only enqueues kernels (append, mask classes, attention): it can be captured, and
+    replays — interleaved with unrelated eager work — reproduce the eager result bit for bit."""
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    B, H, D, L, S, P = 2, 4, 128, 384, 200, 100
+    for dtype in ("f16", "f32"):
+        q, k, v, kc, vc, f = make(B, H, D, L, S, dtype, 17)
+        t = lambda a: torch.from_numpy(a).to(gpu)
+        op = PrefillAttention(B, H, D, L, S, torch.float16 if dtype == "f16" else torch.float32, device=gpu)
+        qd, kd, vd, fd, md = t(q), t(k), t(v), t(f), t(causal_mask(L, -FMAX))
+        kc_d, vc_d = t(kc), t(vc)
+        eager = op.prefill(qd, kd, vd, kc_d, vc_d, fd, start_pos=P, attn_mask=md).clone()
+        out = torch.zeros_like(eager)
+        io = op.make_io(qd, kd, vd, kc_d, vc_d, fd, out, start_pos=P, attn_mask=md)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream(device=gpu)
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(g, stream=side):
+                assert op.launch_prefill(io, S, stream=torch.cuda.current_stream(gpu)) == 0
+        torch.cuda.synchronize()
+        for rep in range(3):
+            out.fill_(float("nan"))
+            _ = (torch.randn(1 << 20, device=gpu) * 2).sum().item()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), f"{dtype} replay {rep}"
+
+
 def test_prefill_literal_rope_rows(gpu):
     # reference as written: token s of the prompt is rotated by table row s (decoder_kernels.cu:440)
     out, want, _ = run_both(gpu, 2, 4, 128, 128, 60, 20, "f32", mask=causal_mask(128), rope_row=0)
