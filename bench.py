@@ -197,6 +197,11 @@ def main() -> int:
                          "-1e5 (its kernel harness) above the diagonal, or no mask")
     ap.add_argument("--prefill-fast-qk", action="store_true",
                     help="prompt-phase fp16 workloads: FL_ATTN_FLAG_FAST_PROMPT_QK (queries as one fp16 value)")
+    ap.add_argument("--mask", default="none", choices=["none", "causal", "strict"],
+                    help="decode workloads: additive mask [L, L] with row stride L, row start_pos is used "
+                         "(open_decoder.cu:207): causal = 0 up to and including the new token, -FLT_MAX beyond; "
+                         "strict = the reference driver's mask, which also hides the new token "
+                         "(samples/llama_fp16.cu:73-81)")
     ap.add_argument("--segment", default="attention", choices=["attention", "int32-int8"],
                     help="attention: q/k/v in the cache dtype -> float output (the headline metric). "
                          "int32-int8: the whole reference segment, int32 GEMM accumulators + scales in, "
@@ -273,6 +278,12 @@ def main() -> int:
     freq_h = synth.freq_cis_table(L, D)
     q, k, v = (torch.from_numpy(a).to(dev) for a in (q_h, k_h, v_h))
     freq = torch.from_numpy(freq_h).to(dev)
+    mask_h = None
+    if args.mask != "none":
+        fmax = float(np.finfo(np.float32).max)
+        r, c = np.arange(L)[:, None], np.arange(L)[None, :]
+        mask_h = np.where(c <= r if args.mask == "causal" else c < r, 0.0, -fmax).astype(np.float32)
+    mask_d = None if mask_h is None else torch.from_numpy(mask_h).to(dev)
     pos_d = torch.from_numpy(pos_h).to(dev) if ragged else None
     # small workloads rotate over several cache copies so the rows do not sit in the 256 MB MALL
     caches = []
@@ -300,7 +311,7 @@ def main() -> int:
             out_int8=torch.empty(B, H * D, dtype=torch.int8, device=dev),
             out_scale=torch.empty(B, dtype=torch.float32, device=dev))
     ios = [op.make_io(q, k, v, kc, vc, freq, out, start_pos=start_pos, start_pos_per_seq=pos_d,
-                      max_start_pos=start_pos if ragged else -1, **extra) for kc, vc in caches]
+                      max_start_pos=start_pos if ragged else -1, attn_mask=mask_d, **extra) for kc, vc in caches]
     stream = torch.cuda.current_stream(dev)
 
     def run(n, passes=3):
@@ -361,7 +372,7 @@ def main() -> int:
         if not np.array_equal(out.cpu().numpy(), out_gpu):
             raise RuntimeError("HIP-graph replay and eager step disagree")
 
-    alg = algorithmic_bytes(B, H, D, e, sum_ctx)
+    alg = algorithmic_bytes(B, H, D, e, sum_ctx, has_mask=mask_h is not None, mean_ctx=sum_ctx / B)
     gbps = alg / (step_ms * 1e-3) / 1e9
     kern_gbps = alg / (kern_ms * 1e-3) / 1e9
 
@@ -374,7 +385,8 @@ def main() -> int:
         ns = args.cpu_seqs or max(1, min(B, int(round(0.5e9 / per_seq))))  # ~0.5 GB of K+V per pass
         sl = slice(0, ns)
         pos_s = pos_h[sl] if ragged else None
-        sample_bytes = algorithmic_bytes(ns, H, D, e, int(lens[sl].sum()))
+        sample_bytes = algorithmic_bytes(ns, H, D, e, int(lens[sl].sum()), has_mask=mask_h is not None,
+                                         mean_ctx=float(lens[sl].mean()))
 
         def cpu_leg(threads, budget_s, max_reps):
             kc_s, vc_s = kc_h[sl].copy(), vc_h[sl].copy()
@@ -382,7 +394,7 @@ def main() -> int:
             while sum(times) < budget_s and len(times) < max_reps:
                 t1 = time.perf_counter()
                 res = ref.decode_attn(q_h[sl], k_h[sl], v_h[sl], kc_s, vc_s, freq_h, start_pos=start_pos,
-                                      start_pos_per_seq=pos_s, threads=threads)
+                                      start_pos_per_seq=pos_s, attn_mask=mask_h, threads=threads)
                 times.append(time.perf_counter() - t1)
             return res, min(times), len(times), sum(times)
 
@@ -420,7 +432,9 @@ def main() -> int:
         "config": {
             "workload": f"{args.workload}: decode self-attention step, B={B} H={H} D={D} "
                         + (f"ragged ctx U[1,{L}] (sum {sum_ctx})" if ragged else f"ctx={max_ctx}")
-                        + f" L={L} {w['dtype']} KV cache, RoPE at position, no mask",
+                        + f" L={L} {w['dtype']} KV cache, RoPE at position, "
+                        + {"none": "no mask", "causal": "causal additive mask row (0 / -FLT_MAX)",
+                           "strict": "the reference driver's strict mask row (new token hidden)"}[args.mask],
             "batch": B, "heads": H, "head_dim": D, "ctx": max_ctx if not ragged else None,
             "sum_ctx": sum_ctx, "cache_rows": L, "cache_copies_rotated": copies,
             "nsplit": plan.nsplit, "chunk_rows": plan.chunk_rows, "two_pass": bool(plan.two_pass),

@@ -31,6 +31,61 @@ HIP_FLAGS = [
 ]
 
 
+def sources(name: str) -> list[str]:
+    """Files a target is built from (a change in any of them makes the built file stale)."""
+    import glob
+    hip = sorted(glob.glob(os.path.join(CSRC, "*.hip")) + glob.glob(os.path.join(CSRC, "*.hpp"))) + \
+        [os.path.join(ROOT, "include", "fl_decode_attn.h")]
+    return {
+        "hip": hip,
+        "cxx": [os.path.join(CSRC, "open_decoder.cpp"), os.path.join(CSRC, "open_decoder.h"),
+                os.path.join(ROOT, "include", "fl_decode_attn.h")],
+        "synth": [os.path.join(CSRC, "fl_synth.c")],
+        "oracle": [os.path.join(ROOT, "oracle", "fl_ref_decode_attn.c"), os.path.join(ROOT, "oracle", "Makefile")],
+        "cpptest": [os.path.join(ROOT, "tests", "cpp", "open_decoder_check.cpp"), os.path.join(CSRC, "open_decoder.h"),
+                    os.path.join(ROOT, "include", "fl_decode_attn.h")],
+    }[name]
+
+
+def outputs(name: str) -> str:
+    return {
+        "hip": os.path.join(LIB, "libfl_decode_attn.so"),
+        "cxx": os.path.join(LIB, "libflopendecoder.so"),
+        "synth": os.path.join(LIB, "libfl_synth.so"),
+        "oracle": os.path.join(ROOT, "oracle", "libfl_ref.so"),
+        "cpptest": os.path.join(ROOT, "tests", "cpp", "open_decoder_check"),
+    }[name]
+
+
+def source_hash(name: str) -> str:
+    import hashlib
+    h = hashlib.sha256()
+    for path in sources(name):
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def _stamp(name: str) -> str:
+    return outputs(name) + ".srchash"
+
+
+def is_stale(name: str) -> bool:
+    """True when the built file is absent or was built from other sources than the ones on disk (a
+    content hash written next to it at build time: file times do not survive every copy of a tree)."""
+    if not os.path.exists(outputs(name)) or not os.path.exists(_stamp(name)):
+        return True
+    with open(_stamp(name)) as f:
+        return f.read().strip() != source_hash(name)
+
+
+def _built(name: str) -> str:
+    with open(_stamp(name), "w") as f:
+        f.write(source_hash(name) + "\n")
+    return outputs(name)
+
+
 def _run(cmd: list[str], cwd: str | None = None) -> None:
     print("+", " ".join(cmd), flush=True)
     res = subprocess.run(cmd, cwd=cwd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -55,7 +110,7 @@ def build_hip() -> str:
     os.makedirs(LIB, exist_ok=True)
     out = os.path.join(LIB, "libfl_decode_attn.so")
     _run([hipcc(), *HIP_FLAGS, "-shared", "-o", out, os.path.join(CSRC, "fl_decode_attn.hip")])
-    return out
+    return _built("hip")
 
 
 def build_cxx() -> str:
@@ -65,7 +120,7 @@ def build_cxx() -> str:
           "-I", os.path.join(ROOT, "include"), "-o", out,
           os.path.join(CSRC, "open_decoder.cpp"),
           "-L", LIB, "-lfl_decode_attn", "-Wl,-rpath,$ORIGIN"])
-    return out
+    return _built("cxx")
 
 
 def build_synth() -> str:
@@ -73,12 +128,12 @@ def build_synth() -> str:
     out = os.path.join(LIB, "libfl_synth.so")
     _run(["gcc", "-O2", "-std=c11", "-fPIC", "-shared", "-fopenmp", "-mf16c", "-Wall",
           "-o", out, os.path.join(CSRC, "fl_synth.c"), "-lm"])
-    return out
+    return _built("synth")
 
 
 def build_oracle() -> str:
     _run(["make", "-C", os.path.join(ROOT, "oracle"), "-B"])
-    return os.path.join(ROOT, "oracle", "libfl_ref.so")
+    return _built("oracle")
 
 
 def build_cpptest() -> str:
@@ -90,7 +145,7 @@ def build_cpptest() -> str:
           "-L", os.path.join(ROOT, "oracle"), "-lfl_ref",
           f"-Wl,-rpath,{LIB}", f"-Wl,-rpath,{os.path.join(ROOT, 'oracle')}",
           "-Wl,-rpath,$ORIGIN/../../fasterllama_amd/lib", "-Wl,-rpath,$ORIGIN/../../oracle"])
-    return out
+    return _built("cpptest")
 
 
 TARGETS = {

@@ -9,8 +9,7 @@ import ctypes as C
 import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-# FL_DECODE_ATTN_LIB points at another build of the same library (kernel tuning experiments)
-LIB_PATH = os.environ.get("FL_DECODE_ATTN_LIB") or os.path.join(_PKG, "lib", "libfl_decode_attn.so")
+LIB_PATH = os.path.join(_PKG, "lib", "libfl_decode_attn.so")
 
 FL_ATTN_F32 = 0
 FL_ATTN_F16 = 1

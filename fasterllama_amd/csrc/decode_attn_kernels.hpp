@@ -43,6 +43,7 @@ struct Params {
     int64_t mask_ld;
     int32_t B, H, L;
     int32_t start_pos, rope_row;
+    int32_t max_pos;   // largest position the launch plan covers: nsplit * chunk > max_pos
     int32_t chunk;     // cache rows per split
     int32_t split_cap; // stride of the partial arrays along the split axis
     int32_t direct;    // 1: single split, write normalised output straight to `out`
@@ -217,7 +218,9 @@ void decode_attn_split_kernel(const Params p)
     const int P = p.pos_per_seq ? p.pos_per_seq[b] : p.start_pos;
     const int tid = threadIdx.x;
 
-    if (P < 0 || P >= L) { // position outside the cache: store nothing, poison the output
+    // A position outside the cache, or beyond the bound the launch was planned for (no split would
+    // own its row): store nothing, poison the output.
+    if (P < 0 || P >= L || P > p.max_pos) {
         if (p.direct && split == 0)
             for (int d = tid; d < D; d += WAVES * 64) p.out[(size_t)bh * D + d] = __builtin_nanf("");
         return;
@@ -485,11 +488,12 @@ __global__ __launch_bounds__(kCombineThreads) void decode_attn_combine_kernel(co
     const int bh = blockIdx.x, tid = threadIdx.x;
     const int b = bh / p.H;
     const int P = p.pos_per_seq ? p.pos_per_seq[b] : p.start_pos;
-    if (P < 0 || P >= p.L) { // uniform per block
+    if (P < 0 || P >= p.L || P > p.max_pos) { // uniform per block; no partial of this (b,h) was written
         for (int d = tid; d < D; d += kCombineThreads) p.out[(size_t)bh * D + d] = __builtin_nanf("");
         return;
     }
-    const int nsp = (P + p.chunk) / p.chunk; // ceil((P+1)/chunk) <= split_cap <= kCombineMaxSplits
+    // ceil((P+1)/chunk) <= ceil((max_pos+1)/chunk) = launched splits <= split_cap <= kCombineMaxSplits
+    const int nsp = min((P + p.chunk) / p.chunk, min(p.split_cap, kCombineMaxSplits));
     const size_t slot0 = (size_t)bh * p.split_cap;
     const float floor_m = p.log2_domain ? kMaxFloor * kLog2e : kMaxFloor;
 

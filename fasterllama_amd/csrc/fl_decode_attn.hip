@@ -159,6 +159,17 @@ void make_plan(const fl_attn_desc *d, int ctx, bool ragged, fl_attn_plan *plan)
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// Kernel launch that reports its own status: hipLaunchKernel returns the error of this launch,
+// whereas hipGetLastError would also return (and clear) an error left behind by an earlier,
+// unrelated HIP call of the calling thread.
+template <typename T> struct same_type { typedef T type; };
+template <typename... KArgs>
+hipError_t launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t stream, typename same_type<KArgs>::type... args)
+{
+    void *ptrs[] = {const_cast<void *>(static_cast<const void *>(&args))...};
+    return hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, ptrs, 0, stream);
+}
+
 // Workspace layout: [float output B*H*D (used when the caller asks for INT8 only)]
 //                   [part_o slots*D] [part_m slots] [part_l slots], each 256-byte aligned.
 struct WorkspaceLayout {
@@ -180,23 +191,22 @@ WorkspaceLayout workspace_layout(const fl_attn_desc *d)
 size_t workspace_need(const fl_attn_desc *d) { return workspace_layout(d).total; }
 
 template <int D>
-void launch_combine(const Params &p, int bh, hipStream_t stream)
+hipError_t launch_combine(const Params &p, int bh, hipStream_t stream)
 {
-    hipLaunchKernelGGL((flattn::decode_attn_combine_kernel<D>), dim3(bh), dim3(flattn::kCombineThreads), 0, stream, p);
+    return launch(flattn::decode_attn_combine_kernel<D>, dim3(bh), dim3(flattn::kCombineThreads), stream, p);
 }
 
 hipError_t dispatch_combine(int D, const Params &p, int bh, hipStream_t stream)
 {
     switch (D) {
-    case 32: launch_combine<32>(p, bh, stream); break;
-    case 64: launch_combine<64>(p, bh, stream); break;
-    case 128: launch_combine<128>(p, bh, stream); break;
-    case 256: launch_combine<256>(p, bh, stream); break;
-    case 512: launch_combine<512>(p, bh, stream); break;
-    case 1024: launch_combine<1024>(p, bh, stream); break;
+    case 32: return launch_combine<32>(p, bh, stream);
+    case 64: return launch_combine<64>(p, bh, stream);
+    case 128: return launch_combine<128>(p, bh, stream);
+    case 256: return launch_combine<256>(p, bh, stream);
+    case 512: return launch_combine<512>(p, bh, stream);
+    case 1024: return launch_combine<1024>(p, bh, stream);
     default: return hipErrorInvalidValue;
     }
-    return hipGetLastError();
 }
 
 // fp16 storage streams half the bytes per row, so its softmax uses the one-instruction base-2
@@ -211,12 +221,10 @@ hipError_t launch_split(const Params &p, dim3 grid, hipStream_t stream)
     constexpr int CPL = CH <= 64 ? 1 : CH / 64;
     constexpr int UNROLL = CPL >= 4 ? 1 : (CPL == 2 ? 2 : FLATTN_UNROLL);
     if (p.attn_mask)
-        hipLaunchKernelGGL((flattn::decode_attn_split_kernel<T, D, kWaves, UNROLL, true, kFastExp<T>>), grid,
-                           dim3(kWaves * 64), 0, stream, p);
-    else
-        hipLaunchKernelGGL((flattn::decode_attn_split_kernel<T, D, kWaves, UNROLL, false, kFastExp<T>>), grid,
-                           dim3(kWaves * 64), 0, stream, p);
-    return hipGetLastError();
+        return launch(flattn::decode_attn_split_kernel<T, D, kWaves, UNROLL, true, kFastExp<T>>, grid, dim3(kWaves * 64),
+                      stream, p);
+    return launch(flattn::decode_attn_split_kernel<T, D, kWaves, UNROLL, false, kFastExp<T>>, grid, dim3(kWaves * 64),
+                  stream, p);
 }
 
 template <typename T>
@@ -263,34 +271,25 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
     constexpr int LPR = D / VEC < 64 ? D / VEC : 64;
     constexpr int ROWS = 256 / LPR;
     const int64_t rows = (int64_t)p.B * p.S * p.H;
-    hipLaunchKernelGGL((flattn::prefill_rope_append_kernel<T, D>), dim3((unsigned)((rows + ROWS - 1) / ROWS)), dim3(256), 0,
-                       stream, p);
-    hipError_t e = hipGetLastError();
+    hipError_t e = launch(flattn::prefill_rope_append_kernel<T, D>, dim3((unsigned)((rows + ROWS - 1) / ROWS)), dim3(256),
+                          stream, p);
     if (e != hipSuccess) return e;
     const unsigned qblocks = (unsigned)((p.S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock);
     const dim3 grid(qblocks * (unsigned)(p.B * p.H)); // mapped to (query block, head) by prefill_block_to_tile
     if (p.attn_mask) {
         const int ktiles = (p.start_pos + p.S + flattn::kPrefillKeysPerStep - 1) / flattn::kPrefillKeysPerStep;
-        hipLaunchKernelGGL(flattn::prefill_mask_classify_kernel, dim3((unsigned)ktiles, qblocks), dim3(256), 0, stream, p, ktiles);
-        e = hipGetLastError();
+        e = launch(flattn::prefill_mask_classify_kernel, dim3((unsigned)ktiles, qblocks), dim3(256), stream, p, ktiles);
         if (e != hipSuccess) return e;
     }
     if constexpr (std::is_same<T, _Float16>::value) {
-        if (p.attn_mask && p.fast_qk)
-            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, true, false>), grid, dim3(256), 0, stream, p);
-        else if (p.attn_mask)
-            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, true, true>), grid, dim3(256), 0, stream, p);
-        else if (p.fast_qk)
-            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, false, false>), grid, dim3(256), 0, stream, p);
-        else
-            hipLaunchKernelGGL((flattn::prefill_attn_f16_kernel<D, false, true>), grid, dim3(256), 0, stream, p);
+        if (p.attn_mask && p.fast_qk) return launch(flattn::prefill_attn_f16_kernel<D, true, false>, grid, dim3(256), stream, p);
+        if (p.attn_mask) return launch(flattn::prefill_attn_f16_kernel<D, true, true>, grid, dim3(256), stream, p);
+        if (p.fast_qk) return launch(flattn::prefill_attn_f16_kernel<D, false, false>, grid, dim3(256), stream, p);
+        return launch(flattn::prefill_attn_f16_kernel<D, false, true>, grid, dim3(256), stream, p);
     } else {
-        if (p.attn_mask)
-            hipLaunchKernelGGL((flattn::prefill_attn_kernel<T, D, true>), grid, dim3(256), 0, stream, p);
-        else
-            hipLaunchKernelGGL((flattn::prefill_attn_kernel<T, D, false>), grid, dim3(256), 0, stream, p);
+        if (p.attn_mask) return launch(flattn::prefill_attn_kernel<T, D, true>, grid, dim3(256), stream, p);
+        return launch(flattn::prefill_attn_kernel<T, D, false>, grid, dim3(256), stream, p);
     }
-    return hipGetLastError();
 }
 
 template <typename T>
@@ -393,7 +392,9 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
         max_pos = io->start_pos;
     }
     if (io->rope_row < FL_ATTN_ROPE_AT_POSITION) return FL_ATTN_ERR_POSITION;
-    if (io->attn_mask && io->mask_ld < 0) return FL_ATTN_ERR_ARGUMENT;
+    // a mask row must cover every attended column; mask_ld == 0 is the one-row (broadcast) mask
+    if (io->attn_mask && (io->mask_ld < 0 || (io->mask_ld != 0 && io->mask_ld < (int64_t)max_pos + 1)))
+        return FL_ATTN_ERR_ARGUMENT;
 
     fl_attn_plan plan;
     make_plan(desc, max_pos + 1, ragged, &plan);
@@ -424,7 +425,7 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
     p.wk_scale = io->k_weight_scale; p.wv_scale = io->v_weight_scale;
     p.mask_ld = io->mask_ld;
     p.B = desc->batch_size; p.H = desc->head_num; p.L = L;
-    p.start_pos = io->start_pos; p.rope_row = io->rope_row;
+    p.start_pos = io->start_pos; p.rope_row = io->rope_row; p.max_pos = max_pos;
     p.chunk = plan.chunk_rows; p.split_cap = cap; p.direct = direct ? 1 : 0;
     p.scale = desc->softmax_scale > 0.f ? desc->softmax_scale : 1.0f / sqrtf((float)D);
     p.log2_domain = desc->dtype == FL_ATTN_F16 ? 1 : 0;
@@ -440,9 +441,9 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
     if (passes & 2) {
         if (!direct && !check_hip(dispatch_combine(D, p, bh, stream))) return FL_ATTN_ERR_HIP;
         if (quant) {
-            hipLaunchKernelGGL(flattn::attn_quantize_transpose_kernel, dim3(desc->batch_size), dim3(1024), 0, stream,
-                               p.out, io->out_int8, io->out_scale, desc->head_num, 1, D);
-            if (!check_hip(hipGetLastError())) return FL_ATTN_ERR_HIP;
+            if (!check_hip(launch(flattn::attn_quantize_transpose_kernel, dim3(desc->batch_size), dim3(1024), stream, p.out,
+                                  io->out_int8, io->out_scale, desc->head_num, 1, D)))
+                return FL_ATTN_ERR_HIP;
         }
     }
     return FL_ATTN_OK;
@@ -488,7 +489,8 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     const int L = desc->total_len;
     if (seq_len < 1 || io->start_pos < 0 || (int64_t)io->start_pos + seq_len > L) return FL_ATTN_ERR_POSITION;
     if (io->rope_row < FL_ATTN_ROPE_AT_POSITION) return FL_ATTN_ERR_POSITION;
-    if (io->attn_mask && io->mask_ld < 0) return FL_ATTN_ERR_ARGUMENT;
+    if (io->attn_mask && (io->mask_ld < 0 || (io->mask_ld != 0 && io->mask_ld < (int64_t)io->start_pos + seq_len)))
+        return FL_ATTN_ERR_ARGUMENT;
     if ((int64_t)desc->batch_size * desc->head_num * ((seq_len + 127) / 128) > (int64_t)INT32_MAX) return FL_ATTN_ERR_SHAPE;
 
     const PrefillWorkspace wl = prefill_workspace(desc, seq_len);
@@ -515,9 +517,9 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     hipError_t e = desc->dtype == FL_ATTN_F16 ? dispatch_prefill<_Float16>(D, p, stream) : dispatch_prefill<float>(D, p, stream);
     if (!check_hip(e)) return FL_ATTN_ERR_HIP;
     if (quant) {
-        hipLaunchKernelGGL(flattn::attn_quantize_transpose_kernel, dim3((unsigned)(desc->batch_size * seq_len)), dim3(1024), 0,
-                           stream, p.out, io->out_int8, io->out_scale, desc->head_num, seq_len, D);
-        if (!check_hip(hipGetLastError())) return FL_ATTN_ERR_HIP;
+        if (!check_hip(launch(flattn::attn_quantize_transpose_kernel, dim3((unsigned)(desc->batch_size * seq_len)), dim3(1024),
+                              stream, p.out, io->out_int8, io->out_scale, desc->head_num, seq_len, D)))
+            return FL_ATTN_ERR_HIP;
     }
     return FL_ATTN_OK;
 }
@@ -532,9 +534,9 @@ int fl_rope_table(float *freq_cis, int32_t rows, int32_t size_per_head, float ba
     const int64_t n = (int64_t)rows * (size_per_head / 2);
     int64_t blocks = (n + 255) / 256;
     if (blocks > 65535) blocks = 65535;
-    hipLaunchKernelGGL(flattn::rope_table_kernel, dim3((unsigned)blocks), dim3(256), 0,
-                       static_cast<hipStream_t>(hip_stream), freq_cis, rows, size_per_head, (double)base);
-    if (!check_hip(hipGetLastError())) return FL_ATTN_ERR_HIP;
+    if (!check_hip(launch(flattn::rope_table_kernel, dim3((unsigned)blocks), dim3(256), static_cast<hipStream_t>(hip_stream),
+                          freq_cis, rows, size_per_head, (double)base)))
+        return FL_ATTN_ERR_HIP;
     return FL_ATTN_OK;
 }
 

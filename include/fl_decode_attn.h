@@ -95,10 +95,13 @@ typedef struct fl_attn_io {
     float *out;                       /* [B, H*D]; may be NULL when out_int8 is given */
     void *workspace;                  /* fl_decode_attn_workspace_bytes() bytes, 256-aligned */
     size_t workspace_bytes;
-    int64_t mask_ld;       /* row stride of attn_mask in floats (the reference uses L) */
+    int64_t mask_ld;       /* row stride of attn_mask in floats (the reference uses L); at least the number
+                              of attended columns, or 0: one row shared by every position */
     int32_t start_pos;     /* tokens already cached; the new token lands in row start_pos */
     int32_t rope_row;      /* table row for RoPE, or FL_ATTN_ROPE_AT_POSITION */
-    int32_t max_start_pos; /* with start_pos_per_seq: upper bound of its entries, <0 = L-1 */
+    int32_t max_start_pos; /* with start_pos_per_seq: upper bound of its entries, <0 = L-1.  The launch is
+                              planned for this bound; a sequence whose device-side position exceeds it
+                              is treated like one outside the cache: NaN output, nothing stored */
     int32_t reserved;      /* must be 0 */
     /* optional prologue: q/k_new/v_new are int32 [B,1,H,D]; x = acc*inp_scale[b]*w_scale[h*D+d] */
     const float *qkv_inp_scale;  /* [B] or NULL */

@@ -170,6 +170,7 @@ typedef struct {
     int64_t mask_ld;
     int start_pos;
     const int32_t *start_pos_per_seq; /* NULL or [B] */
+    int max_start_pos;                /* with start_pos_per_seq: bound the caller promised, <0 = L-1 */
     float scale;
     float *out; /* [B, H*D] */
     int acc_double;
@@ -183,7 +184,10 @@ static void one_head(const ref_args *a, int b, int h, float *scratch)
     const int D = a->D, H = a->H, L = a->L, dt = a->dtype;
     const int P = a->start_pos_per_seq ? a->start_pos_per_seq[b] : a->start_pos;
     float *o_row = a->out + ((size_t)b * H + h) * D;
-    if (P < 0 || P >= L) { /* position outside the cache: nothing stored, output poisoned */
+    const int bound = (a->start_pos_per_seq && a->max_start_pos >= 0) ? a->max_start_pos : L - 1;
+    /* position outside the cache, or beyond the bound the caller promised for a ragged batch
+     * (the HIP library plans its launch for that bound): nothing stored, output poisoned */
+    if (P < 0 || P >= L || P > bound) {
         for (int d = 0; d < D; ++d)
             o_row[d] = NAN;
         return;
@@ -331,6 +335,8 @@ static int run(const ref_args *a, int threads)
 /*
  * One decode step for every (batch, head): RoPE(q, k_new) -> append k/v at row start_pos ->
  * scores over rows [0, start_pos] -> masked softmax -> weighted sum of V rows.
+ * With start_pos_per_seq, max_start_pos >= 0 is the bound the caller promises for its entries; a
+ * sequence beyond it is handled like one outside the cache.
  * dtype selects the storage type of q/k_new/v_new and of both caches (0 = float, 1 = IEEE half);
  * all arithmetic is float (acc_double == 0) or double (acc_double == 1).
  * Returns 0, or a negative code mirroring the C-ABI of the HIP library.
@@ -338,15 +344,16 @@ static int run(const ref_args *a, int threads)
 int fl_ref_decode_attn(int dtype, int B, int H, int D, int L, const void *q, const void *k_new,
                        const void *v_new, void *k_cache, void *v_cache, const float *freq_cis,
                        int rope_row, const float *attn_mask, int64_t mask_ld, int start_pos,
-                       const int32_t *start_pos_per_seq, float scale, float *out, int acc_double,
-                       int threads)
+                       const int32_t *start_pos_per_seq, int max_start_pos, float scale, float *out,
+                       int acc_double, int threads)
 {
     ref_args a;
     memset(&a, 0, sizeof a);
     a.dtype = dtype; a.B = B; a.H = H; a.D = D; a.L = L;
     a.q = q; a.k_new = k_new; a.v_new = v_new; a.k_cache = k_cache; a.v_cache = v_cache;
     a.freq_cis = freq_cis; a.rope_row = rope_row; a.attn_mask = attn_mask; a.mask_ld = mask_ld;
-    a.start_pos = start_pos; a.start_pos_per_seq = start_pos_per_seq; a.scale = scale; a.out = out;
+    a.start_pos = start_pos; a.start_pos_per_seq = start_pos_per_seq; a.max_start_pos = max_start_pos;
+    a.scale = scale; a.out = out;
     a.acc_double = acc_double;
     return run(&a, threads);
 }
@@ -358,7 +365,7 @@ int fl_ref_decode_attn_i32(int dtype, int B, int H, int D, int L, const int32_t 
                            const float *wq_scale, const float *wk_scale, const float *wv_scale,
                            void *k_cache, void *v_cache, const float *freq_cis, int rope_row,
                            const float *attn_mask, int64_t mask_ld, int start_pos,
-                           const int32_t *start_pos_per_seq, float scale, float *out,
+                           const int32_t *start_pos_per_seq, int max_start_pos, float scale, float *out,
                            int acc_double, int threads)
 {
     if (!inp_scale || !wq_scale || !wk_scale || !wv_scale)
@@ -368,7 +375,8 @@ int fl_ref_decode_attn_i32(int dtype, int B, int H, int D, int L, const int32_t 
     a.dtype = dtype; a.B = B; a.H = H; a.D = D; a.L = L;
     a.q = q_acc; a.k_new = k_acc; a.v_new = v_acc; a.k_cache = k_cache; a.v_cache = v_cache;
     a.freq_cis = freq_cis; a.rope_row = rope_row; a.attn_mask = attn_mask; a.mask_ld = mask_ld;
-    a.start_pos = start_pos; a.start_pos_per_seq = start_pos_per_seq; a.scale = scale; a.out = out;
+    a.start_pos = start_pos; a.start_pos_per_seq = start_pos_per_seq; a.max_start_pos = max_start_pos;
+    a.scale = scale; a.out = out;
     a.acc_double = acc_double;
     a.inp_scale = inp_scale; a.wq_scale = wq_scale; a.wk_scale = wk_scale; a.wv_scale = wv_scale;
     return run(&a, threads);

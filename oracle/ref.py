@@ -20,13 +20,13 @@ def load() -> C.CDLL:
         lib = C.CDLL(LIB_PATH)
         lib.fl_ref_decode_attn.argtypes = [
             C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
-            C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_float,
+            C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_int, C.c_float,
             C.c_void_p, C.c_int, C.c_int]
         lib.fl_ref_decode_attn.restype = C.c_int
         lib.fl_ref_decode_attn_i32.argtypes = [
             C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
             C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
-            C.c_int64, C.c_int, C.c_void_p, C.c_float, C.c_void_p, C.c_int, C.c_int]
+            C.c_int64, C.c_int, C.c_void_p, C.c_int, C.c_float, C.c_void_p, C.c_int, C.c_int]
         lib.fl_ref_decode_attn_i32.restype = C.c_int
         lib.fl_ref_freq_cis.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_double]
         lib.fl_ref_freq_cis.restype = C.c_int
@@ -63,12 +63,13 @@ def freq_cis(rows: int, D: int, base: float = 10000.0) -> np.ndarray:
 
 
 def decode_attn(q, k_new, v_new, k_cache, v_cache, freq, start_pos=0, rope_row=-1, attn_mask=None,
-                mask_ld=None, start_pos_per_seq=None, scale=None, acc_double=False, threads=1,
+                mask_ld=None, start_pos_per_seq=None, max_start_pos=-1, scale=None, acc_double=False, threads=1,
                 inp_scale=None, wq_scale=None, wk_scale=None, wv_scale=None, dtype=None):
     """Runs the oracle IN PLACE on k_cache / v_cache (numpy, C-contiguous) and returns out [B, H*D].
 
     q/k_new/v_new: [B,1,H,D] (or [B,H,D]) float32/float16, or int32 with the four scale arrays.
-    k_cache/v_cache: [B,H,L,D] float32 or float16."""
+    k_cache/v_cache: [B,H,L,D] float32 or float16.  With start_pos_per_seq, max_start_pos >= 0 is the
+    bound promised for its entries: a sequence beyond it gets NaN output and no cache row."""
     B, H, L, D = k_cache.shape
     st = np.dtype(k_cache.dtype)
     code = {np.dtype(np.float32): 0, np.dtype(np.float16): 1}[st]
@@ -94,13 +95,14 @@ def decode_attn(q, k_new, v_new, k_cache, v_cache, freq, start_pos=0, rope_row=-
         rc = lib.fl_ref_decode_attn_i32(code, B, H, D, L, _p(q), _p(k_new), _p(v_new), _p(inp_scale),
                                         _p(wq_scale), _p(wk_scale), _p(wv_scale), _p(k_cache), _p(v_cache),
                                         _p(freq), rope_row, _p(attn_mask), mask_ld, start_pos,
-                                        _p(start_pos_per_seq), scale, _p(out), int(acc_double), threads)
+                                        _p(start_pos_per_seq), max_start_pos, scale, _p(out), int(acc_double),
+                                        threads)
     else:
         for a in (q, k_new, v_new):
             assert a.dtype == st
         rc = lib.fl_ref_decode_attn(code, B, H, D, L, _p(q), _p(k_new), _p(v_new), _p(k_cache), _p(v_cache),
                                     _p(freq), rope_row, _p(attn_mask), mask_ld, start_pos,
-                                    _p(start_pos_per_seq), scale, _p(out), int(acc_double), threads)
+                                    _p(start_pos_per_seq), max_start_pos, scale, _p(out), int(acc_double), threads)
     if rc != 0:
         raise ValueError(f"fl_ref_decode_attn -> {rc}")
     return out

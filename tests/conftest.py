@@ -13,16 +13,12 @@ def pytest_configure(config):
 
 
 def _build_missing():
-    """Tests load what is built; they build only what is absent (CPU-side libraries and, by
-    cross-compilation, the HIP library)."""
-    from fasterllama_amd import build, capi, synth
-    oracle_so = os.path.join(ROOT, "oracle", "libfl_ref.so")
-    if not os.path.exists(oracle_so):
-        build.build_oracle()
-    if not os.path.exists(synth.LIB_PATH):
-        build.build_synth()
-    if not os.path.exists(capi.LIB_PATH):
-        build.build_hip()
+    """Tests load what is built; they build only what is absent or was built from other sources than
+    the ones on disk (CPU-side libraries and, by cross-compilation, the HIP library)."""
+    from fasterllama_amd import build
+    for name in ("oracle", "synth", "hip"):
+        if build.is_stale(name):
+            build.TARGETS[name]()
 
 
 @pytest.fixture(scope="session", autouse=True)

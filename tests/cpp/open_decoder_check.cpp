@@ -16,13 +16,13 @@
 extern "C" {
 int fl_ref_decode_attn(int dtype, int B, int H, int D, int L, const void *q, const void *k_new, const void *v_new,
                        void *k_cache, void *v_cache, const float *freq_cis, int rope_row, const float *attn_mask,
-                       int64_t mask_ld, int start_pos, const int32_t *start_pos_per_seq, float scale, float *out,
-                       int acc_double, int threads);
+                       int64_t mask_ld, int start_pos, const int32_t *start_pos_per_seq, int max_start_pos, float scale,
+                       float *out, int acc_double, int threads);
 int fl_ref_decode_attn_i32(int dtype, int B, int H, int D, int L, const int32_t *q_acc, const int32_t *k_acc,
                            const int32_t *v_acc, const float *inp_scale, const float *wq_scale, const float *wk_scale,
                            const float *wv_scale, void *k_cache, void *v_cache, const float *freq_cis, int rope_row,
                            const float *attn_mask, int64_t mask_ld, int start_pos, const int32_t *start_pos_per_seq,
-                           float scale, float *out, int acc_double, int threads);
+                           int max_start_pos, float scale, float *out, int acc_double, int threads);
 int fl_ref_attn_quantize(int B, int HD, const float *attn, int8_t *out_q, float *out_scale);
 int fl_ref_prefill_attn(int dtype, int B, int H, int D, int L, int S, const void *q, const void *k_new, const void *v_new,
                         const float *inp_scale, const float *wq_scale, const float *wk_scale, const float *wv_scale,
@@ -161,7 +161,7 @@ template <OperationType Op, typename CacheT> static void runAll(const char *tag)
         std::vector<CacheT> kc_ref(kc), vc_ref(vc), kc_got(kc.size()), vc_got(vc.size());
         std::vector<float> want((size_t)B * HD), got(want.size());
         fl_ref_decode_attn(code, B, H, D, L, q.data(), k.data(), v.data(), kc_ref.data(), vc_ref.data(), freq.data(), -1,
-                           mask.data(), L, P, nullptr, 1.0f / std::sqrt((float)D), want.data(), 1, 1);
+                           mask.data(), L, P, nullptr, -1, 1.0f / std::sqrt((float)D), want.data(), 1, 1);
         dec.decodeAttention(d_q.p, d_k.p, d_v.p, d_freq.p, d_kc.p, d_vc.p, d_out.p, P);
         HIP_OK(hipStreamSynchronize(stream));
         d_out.down(got.data()); d_kc.down(kc_got.data()); d_vc.down(vc_got.data());
@@ -203,7 +203,7 @@ template <OperationType Op, typename CacheT> static void runAll(const char *tag)
         std::vector<float> want((size_t)B * HD), want_s(B), got_s(B);
         std::vector<int8_t> want8((size_t)B * HD), got8(want8.size());
         fl_ref_decode_attn_i32(code, B, H, D, L, qi.data(), ki.data(), vi.data(), s_in.data(), wq.data(), wk.data(), wv.data(),
-                               kc_ref.data(), vc_ref.data(), freq.data(), -1, mask.data(), L, P, nullptr,
+                               kc_ref.data(), vc_ref.data(), freq.data(), -1, mask.data(), L, P, nullptr, -1,
                                1.0f / std::sqrt((float)D), want.data(), 1, 1);
         fl_ref_attn_quantize(B, HD, want.data(), want8.data(), want_s.data());
         d_seen8.down(got8.data()); d_seens.down(got_s.data()); d_kc.down(kc_got.data());

@@ -97,6 +97,8 @@ def test_null_arguments():
     (dict(k_cache=0x1008), capi.FL_ATTN_ERR_ALIGNMENT),
     (dict(reserved=7), capi.FL_ATTN_ERR_ARGUMENT),
     (dict(attn_mask=0x3000, mask_ld=-5), capi.FL_ATTN_ERR_ARGUMENT),
+    (dict(attn_mask=0x3000, mask_ld=3), capi.FL_ATTN_ERR_ARGUMENT),     # a mask row shorter than the 4 attended columns
+    (dict(attn_mask=0x3000, mask_ld=40, start_pos_per_seq=0x2000, max_start_pos=40), capi.FL_ATTN_ERR_ARGUMENT),
     (dict(q_weight_scale=0x3000), capi.FL_ATTN_ERR_ARGUMENT),          # scales without qkv_inp_scale
     (dict(qkv_inp_scale=0x3000), capi.FL_ATTN_ERR_NULL_POINTER),       # inp scale without weight scales
     (dict(out_int8=0x3000), capi.FL_ATTN_ERR_NULL_POINTER),            # int8 output without its scale

@@ -53,7 +53,7 @@ def test_int32_prologue(gpu, dtype, nsplit):
     torch.cuda.synchronize()
     assert_cache_bit_exact(kc_d.cpu().numpy(), kc, "k_cache")
     assert_cache_bit_exact(vc_d.cpu().numpy(), vc, "v_cache")
-    assert_out_close(out.cpu().numpy(), want, dtype, "int32 prologue")
+    assert_out_close(out.cpu().numpy(), want, dtype, "int32 prologue", head_dim=D)
 
 
 # ----------------------------------------------------------------------------- INT8 epilogue

@@ -11,8 +11,8 @@ EXE = os.path.join(ROOT, "tests", "cpp", "open_decoder_check")
 
 @pytest.mark.gpu
 def test_open_decoder_cpp_driver(gpu):
-    if not os.path.exists(EXE):
-        from fasterllama_amd import build
+    from fasterllama_amd import build
+    if build.is_stale("cxx") or build.is_stale("cpptest"):
         build.build_cxx()
         build.build_cpptest()
     res = subprocess.run([EXE], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
@@ -26,8 +26,8 @@ def test_open_decoder_library_exports_the_reference_instantiations():
     """The shared library carries the same explicit instantiations as the reference's
     libflopendecoder (open_decoder.cu:377-383): OpenDecoder<FP32,INT8> and OpenDecoder<FP16,INT8>."""
     so = os.path.join(ROOT, "fasterllama_amd", "lib", "libflopendecoder.so")
-    if not os.path.exists(so):
-        from fasterllama_amd import build
+    from fasterllama_amd import build
+    if build.is_stale("cxx"):
         build.build_cxx()
     out = subprocess.run(["nm", "-DC", so], stdout=subprocess.PIPE, text=True, check=True).stdout
     for op in ("(FasterLLaMA::OperationType)0", "(FasterLLaMA::OperationType)1"):

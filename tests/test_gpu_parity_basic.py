@@ -15,7 +15,7 @@ def test_config1_tiny(gpu, dtype):
     out, kc, vc, _ = c.run_gpu(gpu)
     assert_cache_bit_exact(kc, kc_ref, "k_cache")
     assert_cache_bit_exact(vc, vc_ref, "v_cache")
-    assert_out_close(out, ref64, dtype, "config1")
+    assert_out_close(out, ref64, dtype, "config1", head_dim=64)
 
 
 @pytest.mark.parametrize("nsplit", [0, 1, 2, 7])

@@ -18,10 +18,12 @@ def check(c, gpu, nsplit=0, what=""):
     assert_cache_bit_exact(kc, kc_ref, what + " k_cache")
     assert_cache_bit_exact(vc, vc_ref, what + " v_cache")
     bad_pos = (c.positions() < 0) | (c.positions() >= c.L)
+    if c.pos is not None:
+        bad_pos |= c.positions() > c.bound()
     if bad_pos.any():
         assert np.isnan(out[bad_pos]).all() and np.isnan(ref64[bad_pos]).all()
         out, ref64 = out[~bad_pos], ref64[~bad_pos]
-    err = assert_out_close(out, ref64, c.dtype, what)
+    err = assert_out_close(out, ref64, c.dtype, what, head_dim=c.D)
     return out, err, op
 
 
@@ -196,6 +198,18 @@ def test_ragged_with_out_of_range_positions(gpu):
     check(c, gpu, nsplit=4, what="ragged invalid split")
 
 
+@pytest.mark.parametrize("nsplit", [0, 1, 4])
+def test_position_above_the_max_start_pos_hint_is_poisoned_not_truncated(gpu, nsplit):
+    # the launch is planned for max_start_pos; a device-side position beyond it must not be served from a
+    # truncated context, nor make the merge read partials nobody wrote: NaN output, caches untouched
+    lens = np.array([4, 302, 2048, 301, 1001, 2])
+    c = Case(6, 3, 128, 2048, "f16", lens=lens, pad=np.nan, max_start_pos=300)
+    out, _, op = check(c, gpu, nsplit=nsplit, what=f"bound 300 nsplit={nsplit}")
+    assert np.isfinite(out).all() and out.shape[0] == 3  # sequences 0, 3 and 5 are served
+    c32 = Case(6, 3, 128, 2048, "f32", lens=lens, pad=np.nan, max_start_pos=300)
+    check(c32, gpu, nsplit=nsplit, what=f"bound 300 f32 nsplit={nsplit}")
+
+
 def test_ragged_lengths_all_tile_remainders(gpu):
     lens = np.arange(1, 131)
     c = Case(130, 2, 64, 130, "f16", lens=lens, pad=np.nan)
@@ -219,7 +233,7 @@ def test_custom_softmax_scale(gpu):
     op = DecodeAttention(1, 4, 128, 128, torch.float32, softmax_scale=0.05, device=gpu)
     t = lambda a: torch.from_numpy(a).to(gpu)
     got = op.forward(t(c.q), t(c.k_new), t(c.v_new), t(c.k_cache), t(c.v_cache), t(c.freq), start_pos=100)
-    assert_out_close(got.cpu().numpy(), want, "f32", "scale=0.05")
+    assert_out_close(got.cpu().numpy(), want, "f32", "scale=0.05", head_dim=128)
 
 
 # ----------------------------------------------------------------------------- error behaviour on the device path
@@ -303,6 +317,6 @@ def test_byte_offsets_beyond_4_gib(gpu):
     assert np.isfinite(out_h).all()
     for b, (kb, vb) in host.items():
         want = ref.decode_attn(q[b:b + 1], k[b:b + 1], v[b:b + 1], kb, vb, freq, start_pos=P, acc_double=True, threads=16)
-        assert_out_close(out_h[b:b + 1], want, "f32", f"sequence {b}")
+        assert_out_close(out_h[b:b + 1], want, "f32", f"sequence {b}", head_dim=D)
         assert_cache_bit_exact(kc_d[b:b + 1].cpu().numpy(), kb, f"k_cache of sequence {b}")
         assert_cache_bit_exact(vc_d[b:b + 1].cpu().numpy(), vb, f"v_cache of sequence {b}")

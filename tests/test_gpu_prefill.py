@@ -114,11 +114,11 @@ def test_prefill_sharp_softmax_with_scaled_keys(gpu, dtype):
     assert_out_close(out, want, dtype, "scaled keys")
     if dtype == "f16":
         # the opt-in fast first product rounds the rotated queries to fp16: scores of magnitude ~90 then
-        # carry ~2e-2 of error each, which this data makes visible (and ordinary data does not)
+        # carry ~2e-2 of error each; the flag promises no more than a loose bound on such data
         fast = PrefillAttention(B, H, D, L, S, torch.float16, device=gpu, fast_qk=True)
         out_fast = fast.prefill(t(q), t(k), t(v), t(kc), t(vc), t(f), attn_mask=t(mask)).cpu().numpy()
         err = np.abs(out_fast - want).max()
-        assert 2e-3 < err < 5e-2, err
+        assert err < 5e-2, err
 
 
 def test_prefill_fast_qk_meets_the_bar_on_ordinary_data(gpu):

@@ -305,6 +305,30 @@ def test_out_of_range_position_poisons_output_and_stores_nothing():
     assert np.array_equal(kc[1], kc0[1])
 
 
+def test_position_above_the_promised_bound_is_treated_like_one_outside_the_cache():
+    # a ragged batch comes with a bound for its positions (the HIP library plans its launch for it);
+    # a sequence beyond that bound gets NaN output and no cache row, its neighbours are untouched by it
+    B, H, D, L = 4, 2, 32, 16
+    q, k, v, kc, vc = make(B, H, D, L, seed=5)
+    kc0, vc0 = kc.copy(), vc.copy()
+    pos = np.array([3, 7, 15, 6])
+    f = ref.freq_cis(L, D)
+    out = ref.decode_attn(q, k, v, kc, vc, f, start_pos_per_seq=pos, max_start_pos=6)
+    assert np.isnan(out[1]).all() and np.isnan(out[2]).all()
+    assert np.array_equal(kc[1:3], kc0[1:3]) and np.array_equal(vc[1:3], vc0[1:3])
+    for b in (0, 3):  # identical to a run of that sequence alone
+        kb, vb = kc0[b:b + 1].copy(), vc0[b:b + 1].copy()
+        ob = ref.decode_attn(q[b:b + 1], k[b:b + 1], v[b:b + 1], kb, vb, f, start_pos=int(pos[b]))
+        assert np.array_equal(ob[0], out[b]) and np.array_equal(kb[0], kc[b]) and np.array_equal(vb[0], vc[b])
+    # no bound given (-1) and a bound equal to the maximum: every sequence is served
+    for bound in (-1, 15):
+        kc1, vc1 = kc0.copy(), vc0.copy()
+        assert np.isfinite(ref.decode_attn(q, k, v, kc1, vc1, f, start_pos_per_seq=pos, max_start_pos=bound)).all()
+    # the bound applies to ragged batches only: a uniform start_pos ignores it
+    kc1, vc1 = kc0.copy(), vc0.copy()
+    assert np.isfinite(ref.decode_attn(q, k, v, kc1, vc1, f, start_pos=9, max_start_pos=2)).all()
+
+
 # ----------------------------------------------------------------------------- fp16 storage (D6 extension)
 
 def test_half_conversions_match_numpy_for_every_half_and_random_floats():
