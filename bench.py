@@ -202,6 +202,9 @@ def main() -> int:
                          "(open_decoder.cu:207): causal = 0 up to and including the new token, -FLT_MAX beyond; "
                          "strict = the reference driver's mask, which also hides the new token "
                          "(samples/llama_fp16.cu:73-81)")
+    ap.add_argument("--two-launches", action="store_true",
+                    help="decode workloads: skip fl_decode_attn_workspace_init, so that a split context is merged "
+                         "by a second launch instead of inside the streaming kernel")
     ap.add_argument("--segment", default="attention", choices=["attention", "int32-int8"],
                     help="attention: q/k/v in the cache dtype -> float output (the headline metric). "
                          "int32-int8: the whole reference segment, int32 GEMM accumulators + scales in, "
@@ -294,6 +297,8 @@ def main() -> int:
     gen_s = time.time() - t0
 
     op = DecodeAttention(B, H, D, L, t_dt, nsplit=args.nsplit, device=dev)
+    if not args.two_launches:
+        op.init_workspace()  # split steps run as one launch (the last workgroup of each (b,h) merges)
     plan = op.plan(max_ctx, ragged)
     extra = {}
     if args.segment == "int32-int8":
@@ -437,7 +442,8 @@ def main() -> int:
                            "strict": "the reference driver's strict mask row (new token hidden)"}[args.mask],
             "batch": B, "heads": H, "head_dim": D, "ctx": max_ctx if not ragged else None,
             "sum_ctx": sum_ctx, "cache_rows": L, "cache_copies_rotated": copies,
-            "nsplit": plan.nsplit, "chunk_rows": plan.chunk_rows, "two_pass": bool(plan.two_pass),
+            "nsplit": plan.nsplit, "chunk_rows": plan.chunk_rows,
+            "launches_per_step": 2 if (plan.two_pass and args.two_launches) else 1,
             "algorithmic_bytes_per_step": alg,
             "segment": args.segment,
         },

@@ -26,6 +26,7 @@ FL_ATTN_ERR_DTYPE = -6
 FL_ATTN_ERR_HIP = -7
 FL_ATTN_ERR_ALIGNMENT = -8
 FL_ATTN_ERR_ARGUMENT = -9
+FL_ATTN_IO_WORKSPACE_READY = 1
 
 # every symbol include/fl_decode_attn.h declares
 EXPORTED_SYMBOLS = (
@@ -33,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "fl_decode_attn_plan",
     "fl_decode_attn_forward",
     "fl_decode_attn_forward_passes",
+    "fl_decode_attn_workspace_init",
     "fl_prefill_attn_workspace_bytes",
     "fl_prefill_attn_forward",
     "fl_rope_table",
@@ -73,7 +75,7 @@ class AttnIO(C.Structure):
         ("start_pos", C.c_int32),
         ("rope_row", C.c_int32),
         ("max_start_pos", C.c_int32),
-        ("reserved", C.c_int32),
+        ("flags", C.c_int32),
         ("qkv_inp_scale", C.c_void_p),
         ("q_weight_scale", C.c_void_p),
         ("k_weight_scale", C.c_void_p),
@@ -121,6 +123,8 @@ def load() -> C.CDLL:
     lib.fl_decode_attn_forward.restype = C.c_int
     lib.fl_decode_attn_forward_passes.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnIO), C.c_void_p, C.c_int]
     lib.fl_decode_attn_forward_passes.restype = C.c_int
+    lib.fl_decode_attn_workspace_init.argtypes = [C.POINTER(AttnDesc), C.c_void_p, C.c_size_t, C.c_void_p]
+    lib.fl_decode_attn_workspace_init.restype = C.c_int
     lib.fl_prefill_attn_workspace_bytes.argtypes = [C.POINTER(AttnDesc), C.c_int32, C.POINTER(C.c_size_t)]
     lib.fl_prefill_attn_workspace_bytes.restype = C.c_int
     lib.fl_prefill_attn_forward.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnIO), C.c_int32, C.c_void_p]

@@ -39,6 +39,7 @@ struct Params {
     float *part_o; // [B*H, split_cap, D]
     float *part_m; // [B*H, split_cap]
     float *part_l; // [B*H, split_cap]
+    int32_t *arrivals; // [B*H] split workgroups that have published their partial; zero between launches
     const float *inp_scale, *wq_scale, *wk_scale, *wv_scale;
     int64_t mask_ld;
     int32_t B, H, L;
@@ -174,6 +175,144 @@ __device__ __forceinline__ void load_token_chunk(const void *base, size_t elem_o
     }
 }
 
+// ---------------------------------------------------------------- merge of split partials
+
+__device__ __forceinline__ float wave_sum(float x)
+{
+    x += dpp_move<0xB1>(x);
+    x += dpp_move<0x4E>(x);
+    x += dpp_move<0x141>(x);
+    x += dpp_move<0x140>(x);
+    x += __shfl_xor(x, 16);
+    x += __shfl_xor(x, 32);
+    return x;
+}
+
+constexpr int kCombineThreads = 256;
+constexpr int kCombineMaxSplits = 1024;
+
+// LDS of one merge: the split weights, two cross-wave reductions and the per-split-group sums.
+template <int D>
+struct CombineShared {
+    static constexpr int TPG = D / 4 < kCombineThreads ? D / 4 : kCombineThreads; // threads per split-group
+    static constexpr int SG = kCombineThreads / TPG;                             // split-groups
+    float w[kCombineMaxSplits];
+    float red[2][kCombineThreads / 64];
+    float4 acc[SG][D / 4];
+};
+
+// Merges the (m, l, o[D]) partials of the first nsp splits of one (b,h), by the 256 threads of a workgroup:
+//   M = max_s m_s;  w_s = exp(m_s - M);  out[d] = sum_s w_s o_s[d] / sum_s w_s l_s.
+// The weights are computed once per split (threads over s), then the weighted sum over splits runs
+// with D/4 threads per split-group (float4 per thread) and 256/(D/4) split-groups side by side, so
+// the partial loads of a group are independent and in flight together.
+template <int D>
+__device__ __forceinline__ void combine_partials(const Params &p, int bh, int nsp, int tid, CombineShared<D> &sh)
+{
+    constexpr int TPG = CombineShared<D>::TPG, SG = CombineShared<D>::SG;
+    constexpr int VPT = D / 4 / TPG; // float4 per thread
+    const size_t slot0 = (size_t)bh * p.split_cap;
+    const float floor_m = p.log2_domain ? kMaxFloor * kLog2e : kMaxFloor;
+
+    float mx = floor_m;
+    for (int s = tid; s < nsp; s += kCombineThreads) {
+        const float ms = p.part_m[slot0 + s];
+        sh.w[s] = ms;
+        mx = fmaxf(mx, ms);
+    }
+    mx = wave_max(mx);
+    if ((tid & 63) == 0) sh.red[0][tid >> 6] = mx;
+    __syncthreads();
+    float M = sh.red[0][0];
+#pragma unroll
+    for (int w = 1; w < kCombineThreads / 64; ++w) M = fmaxf(M, sh.red[0][w]);
+
+    float lsum = 0.f;
+    for (int s = tid; s < nsp; s += kCombineThreads) {
+        const float dm = sh.w[s] - M;
+        const float w = p.log2_domain ? __builtin_amdgcn_exp2f(dm) : expf(dm);
+        sh.w[s] = w;
+        lsum = fmaf(p.part_l[slot0 + s], w, lsum);
+    }
+    lsum = wave_sum(lsum);
+    if ((tid & 63) == 0) sh.red[1][tid >> 6] = lsum;
+    __syncthreads();
+    float Lsum = sh.red[1][0];
+#pragma unroll
+    for (int w = 1; w < kCombineThreads / 64; ++w) Lsum += sh.red[1][w];
+
+    const int sg = tid / TPG, t = tid % TPG;
+    float4 acc[VPT];
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) acc[v] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float4 *po = reinterpret_cast<const float4 *>(p.part_o + slot0 * D);
+    int s = sg;
+    for (; s + 3 * SG < nsp; s += 4 * SG) { // four independent partial rows in flight
+        float4 x[4][VPT];
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int v = 0; v < VPT; ++v) x[k][v] = po[(size_t)(s + k * SG) * (D / 4) + v * TPG + t];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float w = sh.w[s + k * SG];
+#pragma unroll
+            for (int v = 0; v < VPT; ++v) {
+                acc[v].x = fmaf(x[k][v].x, w, acc[v].x);
+                acc[v].y = fmaf(x[k][v].y, w, acc[v].y);
+                acc[v].z = fmaf(x[k][v].z, w, acc[v].z);
+                acc[v].w = fmaf(x[k][v].w, w, acc[v].w);
+            }
+        }
+    }
+    for (; s < nsp; s += SG) {
+        const float w = sh.w[s];
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const float4 x = po[(size_t)s * (D / 4) + v * TPG + t];
+            acc[v].x = fmaf(x.x, w, acc[v].x);
+            acc[v].y = fmaf(x.y, w, acc[v].y);
+            acc[v].z = fmaf(x.z, w, acc[v].z);
+            acc[v].w = fmaf(x.w, w, acc[v].w);
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) sh.acc[sg][v * TPG + t] = acc[v];
+    __syncthreads();
+    for (int d4 = tid; d4 < D / 4; d4 += kCombineThreads) {
+        float4 r = sh.acc[0][d4];
+#pragma unroll
+        for (int k = 1; k < SG; ++k) {
+            const float4 y = sh.acc[k][d4];
+            r.x += y.x; r.y += y.y; r.z += y.z; r.w += y.w;
+        }
+        r.x = r.x / Lsum; r.y = r.y / Lsum; r.z = r.z / Lsum; r.w = r.w / Lsum;
+        reinterpret_cast<float4 *>(p.out + (size_t)bh * D)[d4] = r;
+    }
+}
+
+// Splits of one (b,h) that stream rows (the others return at once): ceil((P+1)/chunk), which is at most
+// ceil((max_pos+1)/chunk) = launched splits <= split_cap <= kCombineMaxSplits.
+__device__ __forceinline__ int active_splits(const Params &p, int P)
+{
+    return min((P + p.chunk) / p.chunk, min(p.split_cap, kCombineMaxSplits));
+}
+
+// grid = B*H, block = 256: the merge as a launch of its own (second pass of a two-pass step).
+template <int D>
+__global__ __launch_bounds__(kCombineThreads) void decode_attn_combine_kernel(const Params p)
+{
+    __shared__ CombineShared<D> sh;
+    const int bh = blockIdx.x, tid = threadIdx.x;
+    const int b = bh / p.H;
+    const int P = p.pos_per_seq ? p.pos_per_seq[b] : p.start_pos;
+    if (P < 0 || P >= p.L || P > p.max_pos) { // uniform per block; no partial of this (b,h) was written
+        for (int d = tid; d < D; d += kCombineThreads) p.out[(size_t)bh * D + d] = __builtin_nanf("");
+        return;
+    }
+    combine_partials<D>(p, bh, active_splits(p, P), tid, sh);
+}
+
 // ---------------------------------------------------------------- streaming (split) kernel
 
 #ifndef FLATTN_MIN_WAVES_PER_EU
@@ -191,7 +330,10 @@ constexpr int min_waves_per_eu()
 }
 
 // FAST selects the base-2 softmax (fp16 storage); the fp32-storage kernels keep expf.
-template <typename T, int D, int WAVES, int UNROLL, bool HAS_MASK, bool FAST>
+// FUSED (split launches only): the workgroup that publishes the last partial of a (b,h) also merges
+// them, so the step is one launch.  Arrivals are counted in p.arrivals[b*H + h], which must be zero
+// when the launch starts and is zero again when it ends.
+template <typename T, int D, int WAVES, int UNROLL, bool HAS_MASK, bool FAST, bool FUSED = false>
 __global__ __launch_bounds__(WAVES * 64)
 __attribute__((amdgpu_waves_per_eu(min_waves_per_eu<T, D>(), 8)))
 void decode_attn_split_kernel(const Params p)
@@ -210,6 +352,9 @@ void decode_attn_split_kernel(const Params p)
     __shared__ float s_o[GROUPS][D];
     __shared__ float s_m[GROUPS];
     __shared__ float s_l[GROUPS];
+    __shared__ typename std::conditional<FUSED, CombineShared<D>, char>::type s_merge;
+    __shared__ int s_last;
+    static_assert(!FUSED || WAVES * 64 == kCombineThreads, "the fused merge runs on a 256-thread workgroup");
 
     const int H = p.H, L = p.L;
     const int BH = p.B * H;
@@ -221,7 +366,7 @@ void decode_attn_split_kernel(const Params p)
     // A position outside the cache, or beyond the bound the launch was planned for (no split would
     // own its row): store nothing, poison the output.
     if (P < 0 || P >= L || P > p.max_pos) {
-        if (p.direct && split == 0)
+        if ((p.direct || FUSED) && split == 0)
             for (int d = tid; d < D; d += WAVES * 64) p.out[(size_t)bh * D + d] = __builtin_nanf("");
         return;
     }
@@ -452,125 +597,26 @@ void decode_attn_split_kernel(const Params p)
             }
         }
     }
-}
 
-// ---------------------------------------------------------------- combine kernels
-
-__device__ __forceinline__ float wave_sum(float x)
-{
-    x += dpp_move<0xB1>(x);
-    x += dpp_move<0x4E>(x);
-    x += dpp_move<0x141>(x);
-    x += dpp_move<0x140>(x);
-    x += __shfl_xor(x, 16);
-    x += __shfl_xor(x, 32);
-    return x;
-}
-
-constexpr int kCombineThreads = 256;
-constexpr int kCombineMaxSplits = 1024;
-
-// grid = B*H, block = 256.  Merges the (m, l, o[D]) partials of one (b,h):
-//   M = max_s m_s;  w_s = exp(m_s - M);  out[d] = sum_s w_s o_s[d] / sum_s w_s l_s.
-// The weights are computed once per split (threads over s), then the weighted sum over splits runs
-// with D/4 threads per split-group (float4 per thread) and 256/(D/4) split-groups side by side, so
-// the partial loads of a group are independent and in flight together.
-template <int D>
-__global__ __launch_bounds__(kCombineThreads) void decode_attn_combine_kernel(const Params p)
-{
-    constexpr int TPG = D / 4 < kCombineThreads ? D / 4 : kCombineThreads; // threads per split-group
-    constexpr int SG = kCombineThreads / TPG;                             // split-groups
-    constexpr int VPT = D / 4 / TPG;                                      // float4 per thread
-    __shared__ float s_w[kCombineMaxSplits];
-    __shared__ float s_red[2][kCombineThreads / 64];
-    __shared__ float4 s_acc[SG][D / 4];
-
-    const int bh = blockIdx.x, tid = threadIdx.x;
-    const int b = bh / p.H;
-    const int P = p.pos_per_seq ? p.pos_per_seq[b] : p.start_pos;
-    if (P < 0 || P >= p.L || P > p.max_pos) { // uniform per block; no partial of this (b,h) was written
-        for (int d = tid; d < D; d += kCombineThreads) p.out[(size_t)bh * D + d] = __builtin_nanf("");
-        return;
-    }
-    // ceil((P+1)/chunk) <= ceil((max_pos+1)/chunk) = launched splits <= split_cap <= kCombineMaxSplits
-    const int nsp = min((P + p.chunk) / p.chunk, min(p.split_cap, kCombineMaxSplits));
-    const size_t slot0 = (size_t)bh * p.split_cap;
-    const float floor_m = p.log2_domain ? kMaxFloor * kLog2e : kMaxFloor;
-
-    float mx = floor_m;
-    for (int s = tid; s < nsp; s += kCombineThreads) {
-        const float ms = p.part_m[slot0 + s];
-        s_w[s] = ms;
-        mx = fmaxf(mx, ms);
-    }
-    mx = wave_max(mx);
-    if ((tid & 63) == 0) s_red[0][tid >> 6] = mx;
-    __syncthreads();
-    float M = s_red[0][0];
-#pragma unroll
-    for (int w = 1; w < kCombineThreads / 64; ++w) M = fmaxf(M, s_red[0][w]);
-
-    float lsum = 0.f;
-    for (int s = tid; s < nsp; s += kCombineThreads) {
-        const float dm = s_w[s] - M;
-        const float w = p.log2_domain ? __builtin_amdgcn_exp2f(dm) : expf(dm);
-        s_w[s] = w;
-        lsum = fmaf(p.part_l[slot0 + s], w, lsum);
-    }
-    lsum = wave_sum(lsum);
-    if ((tid & 63) == 0) s_red[1][tid >> 6] = lsum;
-    __syncthreads();
-    float Lsum = s_red[1][0];
-#pragma unroll
-    for (int w = 1; w < kCombineThreads / 64; ++w) Lsum += s_red[1][w];
-
-    const int sg = tid / TPG, t = tid % TPG;
-    float4 acc[VPT];
-#pragma unroll
-    for (int v = 0; v < VPT; ++v) acc[v] = make_float4(0.f, 0.f, 0.f, 0.f);
-    const float4 *po = reinterpret_cast<const float4 *>(p.part_o + slot0 * D);
-    int s = sg;
-    for (; s + 3 * SG < nsp; s += 4 * SG) { // four independent partial rows in flight
-        float4 x[4][VPT];
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-#pragma unroll
-            for (int v = 0; v < VPT; ++v) x[k][v] = po[(size_t)(s + k * SG) * (D / 4) + v * TPG + t];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const float w = s_w[s + k * SG];
-#pragma unroll
-            for (int v = 0; v < VPT; ++v) {
-                acc[v].x = fmaf(x[k][v].x, w, acc[v].x);
-                acc[v].y = fmaf(x[k][v].y, w, acc[v].y);
-                acc[v].z = fmaf(x[k][v].z, w, acc[v].z);
-                acc[v].w = fmaf(x[k][v].w, w, acc[v].w);
+    if constexpr (FUSED) {
+        if (!p.direct) {
+            // Publish the partial device-wide (the other splits of this (b,h) run on other XCDs, each
+            // behind its own L2), count this workgroup in, and let the last one to arrive merge.
+            __threadfence();
+            __syncthreads();
+            const int nsp = active_splits(p, P);
+            if (tid == 0) {
+                const int before = __hip_atomic_fetch_add(p.arrivals + bh, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+                s_last = before == nsp - 1;
+                if (before == nsp - 1) // every split has arrived: nobody touches the counter again in this launch
+                    __hip_atomic_store(p.arrivals + bh, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            __syncthreads();
+            if (s_last) {
+                __threadfence(); // partial lines this XCD's caches may still hold from an earlier launch are dropped
+                combine_partials<D>(p, bh, nsp, tid, s_merge);
             }
         }
-    }
-    for (; s < nsp; s += SG) {
-        const float w = s_w[s];
-#pragma unroll
-        for (int v = 0; v < VPT; ++v) {
-            const float4 x = po[(size_t)s * (D / 4) + v * TPG + t];
-            acc[v].x = fmaf(x.x, w, acc[v].x);
-            acc[v].y = fmaf(x.y, w, acc[v].y);
-            acc[v].z = fmaf(x.z, w, acc[v].z);
-            acc[v].w = fmaf(x.w, w, acc[v].w);
-        }
-    }
-#pragma unroll
-    for (int v = 0; v < VPT; ++v) s_acc[sg][v * TPG + t] = acc[v];
-    __syncthreads();
-    for (int d4 = tid; d4 < D / 4; d4 += kCombineThreads) {
-        float4 r = s_acc[0][d4];
-#pragma unroll
-        for (int k = 1; k < SG; ++k) {
-            const float4 y = s_acc[k][d4];
-            r.x += y.x; r.y += y.y; r.z += y.z; r.w += y.w;
-        }
-        r.x = r.x / Lsum; r.y = r.y / Lsum; r.z = r.z / Lsum; r.w = r.w / Lsum;
-        reinterpret_cast<float4 *>(p.out + (size_t)bh * D)[d4] = r;
     }
 }
 

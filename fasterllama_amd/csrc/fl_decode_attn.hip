@@ -170,25 +170,37 @@ hipError_t launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t s
     return hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, block, ptrs, 0, stream);
 }
 
-// Workspace layout: [float output B*H*D (used when the caller asks for INT8 only)]
-//                   [part_o slots*D] [part_m slots] [part_l slots], each 256-byte aligned.
+// Workspace layout: [arrivals B*H] [float output B*H*D (used when the caller asks for INT8 only)]
+//                   [part_o slots*D] [part_m slots] [part_l slots], each 256-byte aligned,
+// slots = B*H*cap.  The arrival counters come first so that their place depends on B and H only (not on
+// the cache type or a forced split count).  The caller's workspace is laid out for the largest plan
+// of the shape (cap = split_cap(desc)); the library's own scratch array for the plan of the call.
 struct WorkspaceLayout {
-    size_t tmp_out, part_o, part_m, part_l, total;
+    size_t arrivals, tmp_out, part_o, part_m, part_l, total;
 };
 
-WorkspaceLayout workspace_layout(const fl_attn_desc *d)
+WorkspaceLayout workspace_layout(const fl_attn_desc *d, int cap)
 {
-    const size_t slots = (size_t)d->batch_size * d->head_num * (size_t)split_cap(d);
+    const size_t bh = (size_t)d->batch_size * d->head_num;
+    const size_t slots = bh * (size_t)cap;
     WorkspaceLayout w;
-    w.tmp_out = 0;
-    w.part_o = align_up((size_t)d->batch_size * d->head_num * d->size_per_head * sizeof(float), 256);
+    w.arrivals = 0;
+    w.tmp_out = align_up(bh * sizeof(int32_t), 256);
+    w.part_o = w.tmp_out + align_up(bh * d->size_per_head * sizeof(float), 256);
     w.part_m = w.part_o + align_up(slots * d->size_per_head * sizeof(float), 256);
     w.part_l = w.part_m + align_up(slots * sizeof(float), 256);
     w.total = w.part_l + align_up(slots * sizeof(float), 256);
     return w;
 }
 
+WorkspaceLayout workspace_layout(const fl_attn_desc *d) { return workspace_layout(d, split_cap(d)); }
+
 size_t workspace_need(const fl_attn_desc *d) { return workspace_layout(d).total; }
+
+__global__ void fill_zero_kernel(int32_t *dst, int64_t n)
+{
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) dst[i] = 0;
+}
 
 template <int D>
 hipError_t launch_combine(const Params &p, int bh, hipStream_t stream)
@@ -220,6 +232,14 @@ hipError_t launch_split(const Params &p, dim3 grid, hipStream_t stream)
     constexpr int CH = D / VEC;
     constexpr int CPL = CH <= 64 ? 1 : CH / 64;
     constexpr int UNROLL = CPL >= 4 ? 1 : (CPL == 2 ? 2 : FLATTN_UNROLL);
+    if constexpr (kWaves * 64 == flattn::kCombineThreads) {
+        if (p.arrivals && p.attn_mask) // one launch: the last workgroup of each (b,h) merges the partials
+            return launch(flattn::decode_attn_split_kernel<T, D, kWaves, UNROLL, true, kFastExp<T>, true>, grid,
+                          dim3(kWaves * 64), stream, p);
+        if (p.arrivals)
+            return launch(flattn::decode_attn_split_kernel<T, D, kWaves, UNROLL, false, kFastExp<T>, true>, grid,
+                          dim3(kWaves * 64), stream, p);
+    }
     if (p.attn_mask)
         return launch(flattn::decode_attn_split_kernel<T, D, kWaves, UNROLL, true, kFastExp<T>>, grid, dim3(kWaves * 64),
                       stream, p);
@@ -309,7 +329,7 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 extern "C" {
 
-int fl_attn_version(void) { return 100; }
+int fl_attn_version(void) { return 200; }
 
 int fl_attn_last_hip_error(void) { return g_last_hip_error; }
 
@@ -360,7 +380,14 @@ int fl_decode_attn_plan(const fl_attn_desc *desc, int32_t ctx, int32_t ragged, f
     return FL_ATTN_OK;
 }
 
-int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream, int passes)
+} // extern "C"
+
+namespace {
+
+constexpr bool kFusedMergeBuilt = kWaves * 64 == flattn::kCombineThreads;
+
+// The decode step behind every entry point.
+int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream, int passes)
 {
     int st = validate_desc(desc);
     if (st != FL_ATTN_OK) return st;
@@ -371,7 +398,7 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
     const bool quant = io->out_int8 != nullptr;
     if (!io->out && !quant) return FL_ATTN_ERR_NULL_POINTER;
     if (quant && !io->out_scale) return FL_ATTN_ERR_NULL_POINTER;
-    if (io->reserved != 0) return FL_ATTN_ERR_ARGUMENT;
+    if ((io->flags & ~FL_ATTN_IO_WORKSPACE_READY) != 0) return FL_ATTN_ERR_ARGUMENT;
     const bool i32 = io->qkv_inp_scale != nullptr;
     if (i32 && (!io->q_weight_scale || !io->k_weight_scale || !io->v_weight_scale)) return FL_ATTN_ERR_NULL_POINTER;
     if (!i32 && (io->q_weight_scale || io->k_weight_scale || io->v_weight_scale)) return FL_ATTN_ERR_ARGUMENT;
@@ -403,14 +430,16 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
 
     const bool direct = plan.nsplit == 1; // the streaming kernel normalises and writes the output itself
     const bool need_ws = !direct || (quant && !io->out);
-    const WorkspaceLayout wl = workspace_layout(desc);
+    const WorkspaceLayout wl = workspace_layout(desc, cap);
+    char *ws = static_cast<char *>(io->workspace);
     if (need_ws) {
         if (!io->workspace || io->workspace_bytes < wl.total) return FL_ATTN_ERR_WORKSPACE;
         if ((reinterpret_cast<uintptr_t>(io->workspace) & 255u) != 0) return FL_ATTN_ERR_WORKSPACE;
     }
+    // One launch with the merge inside needs arrival counters that are zero: the caller says so.
+    const bool fused = kFusedMergeBuilt && !direct && passes == 3 && (io->flags & FL_ATTN_IO_WORKSPACE_READY) != 0;
 
     const int D = desc->size_per_head;
-    char *ws = static_cast<char *>(io->workspace);
     Params p{};
     p.q = io->q; p.k_new = io->k_new; p.v_new = io->v_new;
     p.k_cache = io->k_cache; p.v_cache = io->v_cache;
@@ -420,6 +449,7 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
         p.part_o = reinterpret_cast<float *>(ws + wl.part_o);
         p.part_m = reinterpret_cast<float *>(ws + wl.part_m);
         p.part_l = reinterpret_cast<float *>(ws + wl.part_l);
+        if (fused) p.arrivals = reinterpret_cast<int32_t *>(ws + wl.arrivals);
     }
     p.inp_scale = io->qkv_inp_scale; p.wq_scale = io->q_weight_scale;
     p.wk_scale = io->k_weight_scale; p.wv_scale = io->v_weight_scale;
@@ -439,7 +469,7 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
         if (!check_hip(e)) return FL_ATTN_ERR_HIP;
     }
     if (passes & 2) {
-        if (!direct && !check_hip(dispatch_combine(D, p, bh, stream))) return FL_ATTN_ERR_HIP;
+        if (!direct && !fused && !check_hip(dispatch_combine(D, p, bh, stream))) return FL_ATTN_ERR_HIP;
         if (quant) {
             if (!check_hip(launch(flattn::attn_quantize_transpose_kernel, dim3(desc->batch_size), dim3(1024), stream, p.out,
                                   io->out_int8, io->out_scale, desc->head_num, 1, D)))
@@ -449,9 +479,33 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
     return FL_ATTN_OK;
 }
 
+} // namespace
+
+extern "C" {
+
+int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream, int passes)
+{
+    return decode_forward(desc, io, hip_stream, passes);
+}
+
 int fl_decode_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream)
 {
-    return fl_decode_attn_forward_passes(desc, io, hip_stream, 3);
+    return decode_forward(desc, io, hip_stream, 3);
+}
+
+int fl_decode_attn_workspace_init(const fl_attn_desc *desc, void *workspace, size_t workspace_bytes, void *hip_stream)
+{
+    int st = validate_desc(desc);
+    if (st != FL_ATTN_OK) return st;
+    const WorkspaceLayout wl = workspace_layout(desc);
+    if (!workspace || workspace_bytes < wl.total || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
+        return FL_ATTN_ERR_WORKSPACE;
+    const int64_t n = (int64_t)desc->batch_size * desc->head_num;
+    // a fill kernel, not a memset: memset nodes are the one thing a caller cannot safely capture in a HIP graph
+    if (!check_hip(launch(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), static_cast<hipStream_t>(hip_stream),
+                          reinterpret_cast<int32_t *>(static_cast<char *>(workspace) + wl.arrivals), n)))
+        return FL_ATTN_ERR_HIP;
+    return FL_ATTN_OK;
 }
 
 // ---- prompt phase --------------------------------------------------------------------------------
@@ -478,7 +532,7 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     const bool quant = io->out_int8 != nullptr;
     if (!io->out && !quant) return FL_ATTN_ERR_NULL_POINTER;
     if (quant && !io->out_scale) return FL_ATTN_ERR_NULL_POINTER;
-    if (io->reserved != 0 || io->start_pos_per_seq) return FL_ATTN_ERR_ARGUMENT; // uniform positions only
+    if (io->flags != 0 || io->start_pos_per_seq) return FL_ATTN_ERR_ARGUMENT; // uniform positions only
     const bool i32 = io->qkv_inp_scale != nullptr;
     if (i32 && (!io->q_weight_scale || !io->k_weight_scale || !io->v_weight_scale)) return FL_ATTN_ERR_NULL_POINTER;
     if (!i32 && (io->q_weight_scale || io->k_weight_scale || io->v_weight_scale)) return FL_ATTN_ERR_ARGUMENT;

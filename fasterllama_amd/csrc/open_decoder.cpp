@@ -43,10 +43,36 @@ namespace FasterLLaMA
     {
     }
 
+    // Scratch of the decode step: the larger need of the two cache types.
+    template <OperationType OpType_, OperationType QuantizationType>
+    size_t OpenDecoder<OpType_, QuantizationType>::decodeWorkspaceBytes() const
+    {
+        size_t need = 0, x = 0;
+        fl_attn_desc d32 = makeDesc<float>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
+        fl_attn_desc d16 = makeDesc<__half>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
+        throwOnStatus(fl_decode_attn_workspace_bytes(&d32, &x), "getWorkspaceSize");
+        need = x;
+        throwOnStatus(fl_decode_attn_workspace_bytes(&d16, &x), "getWorkspaceSize");
+        return x > need ? x : need;
+    }
+
+    // Scratch of the prompt phase (the same for both cache types); 0 when max_prompt_len is 1.
+    template <OperationType OpType_, OperationType QuantizationType>
+    size_t OpenDecoder<OpType_, QuantizationType>::promptWorkspaceBytes() const
+    {
+        if (max_prompt_len_ <= 1) return 0;
+        size_t x = 0;
+        fl_attn_desc d32 = makeDesc<float>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
+        const int st = fl_prefill_attn_workspace_bytes(&d32, max_prompt_len_, &x);
+        if (st == FL_ATTN_ERR_HEAD_DIM) return 0; // a head size the prompt phase does not serve: forward() reports it
+        throwOnStatus(st, "getWorkspaceSize");
+        return x;
+    }
+
     // Workspace = the buffers of the attention segment for up to batch_size * max_prompt_len tokens, each
     // 256-byte aligned: int8 attention output | activation scales | three int32 accumulator buffers |
-    // output scales | scratch of the attention kernels (the largest need over both cache types and both
-    // phases; the prompt phase is left out when size_per_head is outside its supported set).
+    // output scales | scratch of the decode step | scratch of the prompt phase.  The two scratch areas
+    // are kept apart: the decode area carries arrival counters that must stay zero between steps.
     template <OperationType OpType_, OperationType QuantizationType>
     size_t OpenDecoder<OpType_, QuantizationType>::getWorkspaceSizeBytes() const
     {
@@ -56,16 +82,7 @@ namespace FasterLLaMA
         n += roundUp(tokens * sizeof(float), 256);
         n += 3 * roundUp(tokens * hidden_units_ * sizeof(int32_t), 256);
         n += roundUp(tokens * sizeof(float), 256);
-        size_t need = 0, x = 0;
-        fl_attn_desc d32 = makeDesc<float>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
-        fl_attn_desc d16 = makeDesc<__half>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
-        throwOnStatus(fl_decode_attn_workspace_bytes(&d32, &x), "getWorkspaceSize");
-        need = x;
-        throwOnStatus(fl_decode_attn_workspace_bytes(&d16, &x), "getWorkspaceSize");
-        if (x > need) need = x;
-        if (max_prompt_len_ > 1 && fl_prefill_attn_workspace_bytes(&d32, max_prompt_len_, &x) == FL_ATTN_OK && x > need)
-            need = x; // same for both cache types
-        return n + need + 256; // slack to align a caller's base pointer
+        return n + roundUp(decodeWorkspaceBytes(), 256) + roundUp(promptWorkspaceBytes(), 256) + 256; // slack to align a caller's base pointer
     }
 
     template <OperationType OpType_, OperationType QuantizationType>
@@ -97,7 +114,14 @@ namespace FasterLLaMA
         qkv_buf_ = reinterpret_cast<float *>(p);
         p += roundUp(tokens * sizeof(float), 256);
         attn_workspace_ = p;
-        attn_workspace_bytes_ = getWorkspaceSizeBytes() - (size_t)(p - reinterpret_cast<char *>(roundUp(reinterpret_cast<uintptr_t>(buf), 256))) - 256;
+        attn_workspace_bytes_ = decodeWorkspaceBytes();
+        p += roundUp(attn_workspace_bytes_, 256);
+        prompt_workspace_ = p;
+        prompt_workspace_bytes_ = promptWorkspaceBytes();
+        // arrival counters of the decode scratch start at zero (a small kernel on the caller's stream); from
+        // here on a decode step whose context is split is a single launch
+        fl_attn_desc d = makeDesc<float>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
+        throwOnStatus(fl_decode_attn_workspace_init(&d, attn_workspace_, attn_workspace_bytes_, param_.stream), "initialize");
     }
 
     template <OperationType OpType_, OperationType QuantizationType>
@@ -120,8 +144,9 @@ namespace FasterLLaMA
         io.attn_mask = param_.attn_mask; // row start_pos, stride total_len_ (open_decoder.cu:207)
         io.mask_ld = total_len_;
         io.out = out_float;
-        io.workspace = attn_workspace_;
-        io.workspace_bytes = attn_workspace_bytes_;
+        io.workspace = seq_len == 1 ? attn_workspace_ : prompt_workspace_;
+        io.workspace_bytes = seq_len == 1 ? attn_workspace_bytes_ : prompt_workspace_bytes_;
+        io.flags = seq_len == 1 ? FL_ATTN_IO_WORKSPACE_READY : 0;
         io.start_pos = start_pos;
         io.rope_row = literal_rope_row_ ? 0 : FL_ATTN_ROPE_AT_POSITION;
         io.max_start_pos = -1;

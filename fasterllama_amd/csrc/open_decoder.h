@@ -140,8 +140,13 @@ namespace FasterLLaMA
         int32_t *key_buf_ = nullptr;              // [tokens, hidden]
         int32_t *value_buf_ = nullptr;            // [tokens, hidden]
         float *qkv_buf_ = nullptr;                // [tokens] output scales of the quantised attention output
-        char *attn_workspace_ = nullptr;          // scratch of the attention kernels
+        char *attn_workspace_ = nullptr;          // scratch of the decode-step kernels (split partials, arrival counters)
         size_t attn_workspace_bytes_ = 0;
+        char *prompt_workspace_ = nullptr;        // scratch of the prompt-phase kernels
+        size_t prompt_workspace_bytes_ = 0;
+
+        size_t decodeWorkspaceBytes() const;
+        size_t promptWorkspaceBytes() const;
 
         template <typename CacheT>
         void attentionSegment(const float *freq_cis, CacheT *key_cache, CacheT *value_cache, int start_pos, int seq_len,

@@ -41,6 +41,15 @@ class DecodeAttention:
         self.workspace_bytes = n.value
         # torch allocations are 512-byte aligned; the library asks for 256
         self.workspace = torch.empty(max(n.value, 256), dtype=torch.uint8, device=self.device)
+        self.workspace_ready = False
+
+    def init_workspace(self, stream: torch.cuda.Stream | None = None) -> None:
+        """fl_decode_attn_workspace_init: from here on split steps run as one launch."""
+        s = stream if stream is not None else torch.cuda.current_stream(self.device)
+        with torch.cuda.device(self.device):
+            capi.check(self.lib.fl_decode_attn_workspace_init(C.byref(self.desc), self.workspace.data_ptr(),
+                                                              self.workspace.numel(), C.c_void_p(s.cuda_stream)))
+        self.workspace_ready = True
 
     def plan(self, ctx: int, ragged: bool = False) -> capi.AttnPlan:
         plan = capi.AttnPlan()
@@ -66,7 +75,7 @@ class DecodeAttention:
         io.start_pos = start_pos
         io.rope_row = rope_row
         io.max_start_pos = max_start_pos
-        io.reserved = 0
+        io.flags = capi.FL_ATTN_IO_WORKSPACE_READY if self.workspace_ready else 0
         io.qkv_inp_scale = _ptr(qkv_inp_scale)
         io.q_weight_scale = _ptr(q_weight_scale)
         io.k_weight_scale = _ptr(k_weight_scale)

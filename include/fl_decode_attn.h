@@ -67,6 +67,13 @@ enum { FL_ATTN_F32 = 0, FL_ATTN_F16 = 1 };
  * of a few units and visible (1e-2 on the output) when keys are scaled so that |s| reaches 30-90. */
 #define FL_ATTN_FLAG_FAST_PROMPT_QK 1
 
+/* fl_attn_io.flags.
+ * FL_ATTN_IO_WORKSPACE_READY: the workspace was prepared by fl_decode_attn_workspace_init() and nothing
+ * but this library has written to it since.  A step whose context is split then runs as ONE launch: the
+ * workgroup that finishes the last partial of a (batch, head) pair merges them (otherwise a second,
+ * small launch does). */
+#define FL_ATTN_IO_WORKSPACE_READY 1
+
 /* rope_row value meaning "rotate by the table row of each sequence's own position" */
 #define FL_ATTN_ROPE_AT_POSITION (-1)
 
@@ -102,7 +109,7 @@ typedef struct fl_attn_io {
     int32_t max_start_pos; /* with start_pos_per_seq: upper bound of its entries, <0 = L-1.  The launch is
                               planned for this bound; a sequence whose device-side position exceeds it
                               is treated like one outside the cache: NaN output, nothing stored */
-    int32_t reserved;      /* must be 0 */
+    int32_t flags;         /* 0, or FL_ATTN_IO_ values */
     /* optional prologue: q/k_new/v_new are int32 [B,1,H,D]; x = acc*inp_scale[b]*w_scale[h*D+d] */
     const float *qkv_inp_scale;  /* [B] or NULL */
     const float *q_weight_scale; /* [H*D] */
@@ -138,6 +145,13 @@ int fl_decode_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, void 
  * benchmark time the bandwidth-bound kernel alone; fl_decode_attn_forward == passes 3. */
 int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream,
                                   int passes);
+
+/* Prepares a workspace for steps that carry FL_ATTN_IO_WORKSPACE_READY: zeroes its arrival counters (a small
+ * kernel on the given stream; capturable).  Once per workspace, e.g. where OpenDecoder::initialize carves
+ * its buffers (open_decoder.cu:31-45); every later step leaves the counters zero again.  A step that was
+ * torn down half way (device reset) needs a new call. */
+int fl_decode_attn_workspace_init(const fl_attn_desc *desc, void *workspace, size_t workspace_bytes,
+                                  void *hip_stream);
 
 /* ---- prompt phase (seq_len > 1): the dense branch of the same block -------------------------------
  * Replaces, for seq_len new tokens per sequence at positions start_pos .. start_pos+seq_len-1

@@ -56,17 +56,26 @@ class Case:
                               max_start_pos=self.bound(), acc_double=acc_double, threads=threads)
         return out, kc, vc
 
-    def run_gpu(self, device, nsplit=0, want_passes=3):
+    def run_gpu(self, device, nsplit=0, entry="forward", op=None):
+        """entry: "forward" (fl_decode_attn_forward, two launches when the context is split) or "ready"
+        (the same after fl_decode_attn_workspace_init: one launch).  op: reuse an operator (and its workspace)
+        of the same shape."""
         import torch
+        from fasterllama_amd import capi
         from fasterllama_amd.decode_attn import DecodeAttention
         tdt = torch.float16 if self.dtype == "f16" else torch.float32
-        op = DecodeAttention(self.B, self.H, self.D, self.L, tdt, nsplit=nsplit, device=device)
+        if op is None:
+            op = DecodeAttention(self.B, self.H, self.D, self.L, tdt, nsplit=nsplit, device=device)
+            if entry == "ready":
+                op.init_workspace()
         d = lambda a: None if a is None else torch.from_numpy(a).to(device)
         q, k, v = d(self.q), d(self.k_new), d(self.v_new)
         kc, vc = d(self.k_cache), d(self.v_cache)
         f, m, pos = d(self.freq), d(self.mask), d(self.pos)
-        out = op.forward(q, k, v, kc, vc, f, start_pos=self.start_pos, rope_row=self.rope_row,
-                         attn_mask=m, start_pos_per_seq=pos, max_start_pos=self.bound())
+        out = torch.full((self.B, self.H * self.D), 7.0, dtype=torch.float32, device=device)
+        io = op.make_io(q, k, v, kc, vc, f, out, start_pos=self.start_pos, rope_row=self.rope_row,
+                        attn_mask=m, start_pos_per_seq=pos, max_start_pos=self.bound())
+        capi.check(op.launch(io))
         torch.cuda.synchronize(device)
         return out.cpu().numpy(), kc.cpu().numpy(), vc.cpu().numpy(), op
 

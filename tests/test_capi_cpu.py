@@ -95,7 +95,7 @@ def test_null_arguments():
     (dict(start_pos_per_seq=0x2000, max_start_pos=64), capi.FL_ATTN_ERR_POSITION),
     (dict(q=0x1004), capi.FL_ATTN_ERR_ALIGNMENT),
     (dict(k_cache=0x1008), capi.FL_ATTN_ERR_ALIGNMENT),
-    (dict(reserved=7), capi.FL_ATTN_ERR_ARGUMENT),
+    (dict(flags=6), capi.FL_ATTN_ERR_ARGUMENT),                          # unknown io flag bits
     (dict(attn_mask=0x3000, mask_ld=-5), capi.FL_ATTN_ERR_ARGUMENT),
     (dict(attn_mask=0x3000, mask_ld=3), capi.FL_ATTN_ERR_ARGUMENT),     # a mask row shorter than the 4 attended columns
     (dict(attn_mask=0x3000, mask_ld=40, start_pos_per_seq=0x2000, max_start_pos=40), capi.FL_ATTN_ERR_ARGUMENT),

@@ -12,9 +12,9 @@ from oracle import ref
 pytestmark = pytest.mark.gpu
 
 
-def check(c, gpu, nsplit=0, what=""):
+def check(c, gpu, nsplit=0, what="", entry="forward", op=None):
     ref64, kc_ref, vc_ref = c.run_oracle(acc_double=True, threads=16)
-    out, kc, vc, op = c.run_gpu(gpu, nsplit=nsplit)
+    out, kc, vc, op = c.run_gpu(gpu, nsplit=nsplit, entry=entry, op=op)
     assert_cache_bit_exact(kc, kc_ref, what + " k_cache")
     assert_cache_bit_exact(vc, vc_ref, what + " v_cache")
     bad_pos = (c.positions() < 0) | (c.positions() >= c.L)
@@ -62,6 +62,43 @@ def test_config2_fp32_cache_variant(gpu):
     # the reference's own cache type (float) at the LLaMA2-7B shape
     c = Case(8, 32, 128, 1024, "f32", start_pos=1023)
     check(c, gpu, what="config2 f32")
+
+
+# ----------------------------------------------------------------------------- one-launch steps (merge inside the streaming kernel)
+
+@pytest.mark.parametrize("nsplit", [0, 2, 7, 64])
+def test_config4_one_launch_equals_two_launches_bitwise(gpu, nsplit):
+    # after fl_decode_attn_workspace_init the last workgroup of each (b,h) merges the partials: the same
+    # arithmetic in the same order as the combine launch, so the outputs agree bit for bit
+    c = Case(1, 32, 128, 4096, "f16", start_pos=4095, scale_rows=(17, 1000, 4000))
+    two = c.run_gpu(gpu, nsplit=nsplit)[0]
+    one, _, op = check(c, gpu, nsplit=nsplit, what=f"config4 one launch nsplit={nsplit}", entry="ready")
+    assert op.plan(4096).nsplit > 1
+    assert np.array_equal(one, two)
+    # the arrival counters are back at zero: the same workspace serves further steps, also other contexts
+    for ctx in (4096, 1000, 65, 4096):
+        c2 = Case(1, 32, 128, 4096, "f16", start_pos=ctx - 1, seed=ctx)
+        check(c2, gpu, what=f"one launch, reused workspace, ctx={ctx}", entry="ready", op=op)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_one_launch_ragged_masks_and_invalid_positions(gpu, dtype):
+    B, L = 7, 1024
+    lens = np.array([1, 1024, 0, 333, 1025, 64, 65])  # positions -1 and 1024 are invalid
+    m = (np.random.default_rng(3).standard_normal((L, L)) * 2).astype(np.float32)
+    c = Case(B, 5, 128, L, dtype, lens=lens, pad=np.nan, mask=m)
+    _, _, op = check(c, gpu, nsplit=6, what="one launch ragged", entry="ready")
+    check(c, gpu, what="one launch ragged, again", entry="ready", op=op)
+    lens2 = np.array([4, 302, 1024, 301, 1001, 2, 300])
+    c2 = Case(B, 5, 128, L, dtype, lens=lens2, pad=np.nan, max_start_pos=300)
+    check(c2, gpu, what="one launch, bound 300", entry="ready", op=op)
+
+
+@pytest.mark.parametrize("D", [32, 64, 256, 512, 1024])
+def test_one_launch_head_sizes(gpu, D):
+    for dtype in ("f16", "f32"):
+        c = Case(2, 2, D, 300, dtype, start_pos=277, seed=D)
+        check(c, gpu, nsplit=3, what=f"one launch D={D} {dtype}", entry="ready")
 
 
 # ----------------------------------------------------------------------------- context lengths around tile edges
