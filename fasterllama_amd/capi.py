@@ -26,7 +26,9 @@ FL_ATTN_ERR_DTYPE = -6
 FL_ATTN_ERR_HIP = -7
 FL_ATTN_ERR_ALIGNMENT = -8
 FL_ATTN_ERR_ARGUMENT = -9
+FL_ATTN_ERR_SCRATCH_LIMIT = -10
 FL_ATTN_IO_WORKSPACE_READY = 1
+FL_ATTN_NOALLOC_SCRATCH_BYTES = 16 << 20
 
 # every symbol include/fl_decode_attn.h declares
 EXPORTED_SYMBOLS = (
@@ -34,6 +36,7 @@ EXPORTED_SYMBOLS = (
     "fl_decode_attn_plan",
     "fl_decode_attn_forward",
     "fl_decode_attn_forward_passes",
+    "fl_decode_attn_forward_noalloc",
     "fl_decode_attn_workspace_init",
     "fl_prefill_attn_workspace_bytes",
     "fl_prefill_attn_forward",
@@ -123,6 +126,8 @@ def load() -> C.CDLL:
     lib.fl_decode_attn_forward.restype = C.c_int
     lib.fl_decode_attn_forward_passes.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnIO), C.c_void_p, C.c_int]
     lib.fl_decode_attn_forward_passes.restype = C.c_int
+    lib.fl_decode_attn_forward_noalloc.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnIO), C.c_void_p]
+    lib.fl_decode_attn_forward_noalloc.restype = C.c_int
     lib.fl_decode_attn_workspace_init.argtypes = [C.POINTER(AttnDesc), C.c_void_p, C.c_size_t, C.c_void_p]
     lib.fl_decode_attn_workspace_init.restype = C.c_int
     lib.fl_prefill_attn_workspace_bytes.argtypes = [C.POINTER(AttnDesc), C.c_int32, C.POINTER(C.c_size_t)]

@@ -197,6 +197,34 @@ WorkspaceLayout workspace_layout(const fl_attn_desc *d) { return workspace_layou
 
 size_t workspace_need(const fl_attn_desc *d) { return workspace_layout(d).total; }
 
+// Scratch memory of fl_decode_attn_forward_noalloc: one array per GPU, part of the library's code
+// object, so that entry point never allocates.  Static storage starts out zero, which is the state the
+// arrival counters need, and every launch that uses them leaves them zero again.
+constexpr size_t kScratchBytes = FL_ATTN_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char g_scratch[kScratchBytes];
+
+// Device address of g_scratch on the current device (each GPU holds its own copy at its own address);
+// looked up once per device.  In host code the array's name is only a handle for this lookup.
+hipError_t scratch_address(char **ptr)
+{
+    static std::atomic<char *> cached[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    char *p = cached[dev].load(std::memory_order_acquire);
+    if (!p) {
+        void *sym = nullptr;
+        e = hipGetSymbolAddress(&sym, HIP_SYMBOL(g_scratch));
+        if (e != hipSuccess) return e;
+        if (!sym) return hipErrorInvalidSymbol;
+        p = static_cast<char *>(sym);
+        cached[dev].store(p, std::memory_order_release);
+    }
+    *ptr = p;
+    return hipSuccess;
+}
+
 __global__ void fill_zero_kernel(int32_t *dst, int64_t n)
 {
     for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) dst[i] = 0;
@@ -347,6 +375,9 @@ const char *fl_attn_strerror(int status)
     case FL_ATTN_ERR_HIP: return "a HIP runtime call failed";
     case FL_ATTN_ERR_ALIGNMENT: return "tensor base pointers must be 16-byte aligned";
     case FL_ATTN_ERR_ARGUMENT: return "inconsistent arguments";
+    case FL_ATTN_ERR_SCRATCH_LIMIT:
+        return "the step needs more scratch than fl_decode_attn_forward_noalloc holds (FL_ATTN_NOALLOC_SCRATCH_BYTES); "
+               "use fl_decode_attn_forward with a caller-owned workspace";
     default: return "unknown status";
     }
 }
@@ -386,8 +417,9 @@ namespace {
 
 constexpr bool kFusedMergeBuilt = kWaves * 64 == flattn::kCombineThreads;
 
-// The decode step behind every entry point.
-int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream, int passes)
+// The decode step behind every entry point.  own_scratch: take the split partials and arrival
+// counters from the library's per-GPU scratch array instead of io->workspace (no allocation either way).
+int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream, int passes, bool own_scratch)
 {
     int st = validate_desc(desc);
     if (st != FL_ATTN_OK) return st;
@@ -425,19 +457,27 @@ int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_str
 
     fl_attn_plan plan;
     make_plan(desc, max_pos + 1, ragged, &plan);
-    const int cap = split_cap(desc);
+    const int cap = own_scratch ? plan.nsplit : split_cap(desc);
     if (plan.nsplit > cap) return FL_ATTN_ERR_ARGUMENT;
 
     const bool direct = plan.nsplit == 1; // the streaming kernel normalises and writes the output itself
     const bool need_ws = !direct || (quant && !io->out);
     const WorkspaceLayout wl = workspace_layout(desc, cap);
     char *ws = static_cast<char *>(io->workspace);
-    if (need_ws) {
+    if (own_scratch) {
+        ws = nullptr;
+        if (need_ws) {
+            if (wl.total > kScratchBytes) return FL_ATTN_ERR_SCRATCH_LIMIT;
+            if (!check_hip(scratch_address(&ws))) return FL_ATTN_ERR_HIP;
+        }
+    } else if (need_ws) {
         if (!io->workspace || io->workspace_bytes < wl.total) return FL_ATTN_ERR_WORKSPACE;
         if ((reinterpret_cast<uintptr_t>(io->workspace) & 255u) != 0) return FL_ATTN_ERR_WORKSPACE;
     }
-    // One launch with the merge inside needs arrival counters that are zero: the caller says so.
-    const bool fused = kFusedMergeBuilt && !direct && passes == 3 && (io->flags & FL_ATTN_IO_WORKSPACE_READY) != 0;
+    // One launch with the merge inside needs arrival counters that are zero: the library's own scratch
+    // always is (between launches), the caller's workspace when it says so.
+    const bool fused = kFusedMergeBuilt && !direct && passes == 3 &&
+                       (own_scratch || (io->flags & FL_ATTN_IO_WORKSPACE_READY) != 0);
 
     const int D = desc->size_per_head;
     Params p{};
@@ -485,12 +525,17 @@ extern "C" {
 
 int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream, int passes)
 {
-    return decode_forward(desc, io, hip_stream, passes);
+    return decode_forward(desc, io, hip_stream, passes, false);
 }
 
 int fl_decode_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream)
 {
-    return decode_forward(desc, io, hip_stream, 3);
+    return decode_forward(desc, io, hip_stream, 3, false);
+}
+
+int fl_decode_attn_forward_noalloc(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream)
+{
+    return decode_forward(desc, io, hip_stream, 3, true);
 }
 
 int fl_decode_attn_workspace_init(const fl_attn_desc *desc, void *workspace, size_t workspace_bytes, void *hip_stream)

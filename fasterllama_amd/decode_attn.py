@@ -91,6 +91,12 @@ class DecodeAttention:
             return self.lib.fl_decode_attn_forward_passes(C.byref(self.desc), C.byref(io),
                                                           C.c_void_p(s.cuda_stream), passes)
 
+    def launch_noalloc(self, io: capi.AttnIO, stream: torch.cuda.Stream | None = None) -> int:
+        """Same step through fl_decode_attn_forward_noalloc (the library's own scratch array)."""
+        s = stream if stream is not None else torch.cuda.current_stream(self.device)
+        with torch.cuda.device(self.device):
+            return self.lib.fl_decode_attn_forward_noalloc(C.byref(self.desc), C.byref(io), C.c_void_p(s.cuda_stream))
+
     def forward(self, q, k_new, v_new, k_cache, v_cache, freq_cis, start_pos: int = 0, out=None, **kw):
         """RoPE(q, k_new) -> append k/v at row start_pos -> attention over rows [0, start_pos].
 

@@ -55,7 +55,9 @@ typedef enum fl_attn_status {
     FL_ATTN_ERR_DTYPE = -6,         /* dtype is neither FL_ATTN_F32 nor FL_ATTN_F16 */
     FL_ATTN_ERR_HIP = -7,           /* a HIP runtime call failed (see fl_attn_last_hip_error) */
     FL_ATTN_ERR_ALIGNMENT = -8,     /* a tensor base is not 16-byte aligned */
-    FL_ATTN_ERR_ARGUMENT = -9       /* inconsistent optional arguments */
+    FL_ATTN_ERR_ARGUMENT = -9,      /* inconsistent optional arguments */
+    FL_ATTN_ERR_SCRATCH_LIMIT = -10 /* fl_decode_attn_forward_noalloc: the step needs more scratch than
+                                       FL_ATTN_NOALLOC_SCRATCH_BYTES */
 } fl_attn_status;
 
 enum { FL_ATTN_F32 = 0, FL_ATTN_F16 = 1 };
@@ -73,6 +75,9 @@ enum { FL_ATTN_F32 = 0, FL_ATTN_F16 = 1 };
  * workgroup that finishes the last partial of a (batch, head) pair merges them (otherwise a second,
  * small launch does). */
 #define FL_ATTN_IO_WORKSPACE_READY 1
+
+/* Bytes of device scratch fl_decode_attn_forward_noalloc holds per GPU. */
+#define FL_ATTN_NOALLOC_SCRATCH_BYTES (16u << 20)
 
 /* rope_row value meaning "rotate by the table row of each sequence's own position" */
 #define FL_ATTN_ROPE_AT_POSITION (-1)
@@ -152,6 +157,20 @@ int fl_decode_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io
  * torn down half way (device reset) needs a new call. */
 int fl_decode_attn_workspace_init(const fl_attn_desc *desc, void *workspace, size_t workspace_bytes,
                                   void *hip_stream);
+
+/* fl_decode_attn_forward for callers that cannot allocate or hand over device memory at the point of the
+ * call (code under HIP-graph capture, tight serving loops, harnesses that forbid hipMalloc): the split
+ * partials and arrival counters live in an array of FL_ATTN_NOALLOC_SCRATCH_BYTES that is part of the
+ * library's code object (one copy per GPU, held until the process ends) instead of io->workspace, which is
+ * ignored together with io->workspace_bytes and FL_ATTN_IO_WORKSPACE_READY.  No counterpart in the
+ * reference, whose forward() works in the buffer carved at initialize().  Same operands, results and status
+ * codes as fl_decode_attn_forward, plus FL_ATTN_ERR_SCRATCH_LIMIT when the plan of the step needs more than
+ * the array holds (B * H * splits * (D + 2) * 4 bytes and B * H counters; nothing when the context is not
+ * split and a float output is given).  Split steps run as one launch.  Every call on a GPU shares that
+ * GPU's array: calls that may run at the same time on one GPU (two streams, two threads) race; calls in
+ * stream order do not.  The first call on each GPU also looks up the array's device address
+ * (hipGetSymbolAddress): make that call outside stream capture. */
+int fl_decode_attn_forward_noalloc(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream);
 
 /* ---- prompt phase (seq_len > 1): the dense branch of the same block -------------------------------
  * Replaces, for seq_len new tokens per sequence at positions start_pos .. start_pos+seq_len-1

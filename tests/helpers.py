@@ -57,9 +57,9 @@ class Case:
         return out, kc, vc
 
     def run_gpu(self, device, nsplit=0, entry="forward", op=None):
-        """entry: "forward" (fl_decode_attn_forward, two launches when the context is split) or "ready"
-        (the same after fl_decode_attn_workspace_init: one launch).  op: reuse an operator (and its workspace)
-        of the same shape."""
+        """entry: "forward" (fl_decode_attn_forward, two launches when the context is split), "ready"
+        (the same after fl_decode_attn_workspace_init: one launch) or "noalloc"
+        (fl_decode_attn_forward_noalloc).  op: reuse an operator (and its workspace) of the same shape."""
         import torch
         from fasterllama_amd import capi
         from fasterllama_amd.decode_attn import DecodeAttention
@@ -75,7 +75,11 @@ class Case:
         out = torch.full((self.B, self.H * self.D), 7.0, dtype=torch.float32, device=device)
         io = op.make_io(q, k, v, kc, vc, f, out, start_pos=self.start_pos, rope_row=self.rope_row,
                         attn_mask=m, start_pos_per_seq=pos, max_start_pos=self.bound())
-        capi.check(op.launch(io))
+        if entry == "noalloc":
+            io.workspace, io.workspace_bytes = None, 0
+            capi.check(op.launch_noalloc(io))
+        else:
+            capi.check(op.launch(io))
         torch.cuda.synchronize(device)
         return out.cpu().numpy(), kc.cpu().numpy(), vc.cpu().numpy(), op
 

@@ -46,8 +46,8 @@ def test_struct_layouts_match_the_header():
 
 
 def test_strerror_covers_every_status():
-    msgs = {capi.strerror(s) for s in range(0, -10, -1)}
-    assert len(msgs) == 10 and "unknown status" not in msgs
+    msgs = {capi.strerror(s) for s in range(0, -11, -1)}
+    assert len(msgs) == 11 and "unknown status" not in msgs
     assert capi.strerror(-99) == "unknown status"
 
 

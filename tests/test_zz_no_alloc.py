@@ -1,0 +1,54 @@
+"""fl_decode_attn_forward_noalloc — the entry point that uses the library's own per-GPU scratch array
+instead of a caller workspace — against fl_decode_attn_forward on the same inputs, through the C ABI."""
+import numpy as np
+import pytest
+
+from fasterllama_amd import capi
+from helpers import Case, assert_cache_bit_exact, assert_out_close
+
+pytestmark = pytest.mark.gpu
+
+
+def both(c, gpu, nsplit=0):
+    want, kc_w, vc_w, op = c.run_gpu(gpu, nsplit=nsplit, entry="forward")
+    got, kc_g, vc_g, _ = c.run_gpu(gpu, nsplit=nsplit, entry="noalloc")
+    assert_cache_bit_exact(kc_g, kc_w, "k_cache")
+    assert_cache_bit_exact(vc_g, vc_w, "v_cache")
+    # same kernels, same arithmetic, same order: bit-identical, which is inside any tolerance
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    ref64 = c.run_oracle(acc_double=True, threads=16)[0]
+    ok = ~np.isnan(ref64).any(axis=1)
+    assert_out_close(got[ok], ref64[ok], c.dtype, "noalloc vs oracle", head_dim=c.D)
+    return op
+
+
+def test_noalloc_two_calls_in_a_row_the_second_smaller(gpu):
+    # split context (partials and arrival counters in the scratch array), then a smaller problem that
+    # reuses the same array, then the first again
+    big = Case(1, 32, 128, 4096, "f16", start_pos=4095, scale_rows=(17, 1000, 4000))
+    op = both(big, gpu)
+    assert op.plan(4096).nsplit > 1
+    small = Case(1, 8, 128, 4096, "f16", start_pos=700, seed=5)
+    both(small, gpu)
+    both(big, gpu)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_noalloc_ragged_forced_splits_and_unsplit(gpu, dtype):
+    lens = np.array([1, 512, 0, 333, 513, 64])
+    both(Case(6, 3, 128, 512, dtype, lens=lens, pad=np.nan), gpu, nsplit=5)
+    both(Case(2, 4, 64, 256, dtype, start_pos=100), gpu, nsplit=1)  # no scratch needed at all
+
+
+def test_noalloc_rejects_what_does_not_fit(gpu):
+    import ctypes as C
+    import torch
+    from fasterllama_amd.decode_attn import DecodeAttention
+    # B*H = 4096 pairs x 64 forced splits x (128 + 2) floats = 136 MB of partials > 16 MiB
+    B, H, D, L = 128, 32, 128, 4096
+    op = DecodeAttention(B, H, D, L, torch.float16, nsplit=64, device=gpu)
+    x = torch.zeros(16, dtype=torch.float16, device=gpu)  # never dereferenced: validation fails first
+    io = op.make_io(x, x, x, x, x, x.float(), x.float(), start_pos=L - 1)
+    io.workspace, io.workspace_bytes = None, 0
+    st = op.launch_noalloc(io)
+    assert st == capi.FL_ATTN_ERR_SCRATCH_LIMIT and "scratch" in capi.strerror(st)
