@@ -128,6 +128,21 @@ template <> struct Vec16<_Float16> {
     typedef _Float16 type __attribute__((ext_vector_type(8)));
 };
 
+// Raw buffer loads: address = base (in a 128-bit descriptor held in scalar registers) + a scalar byte
+// offset + a 32-bit per-lane byte offset (+ an immediate).  The streaming loop needs no 64-bit vector
+// address arithmetic and no register pairs for addresses, whatever the compiler's addressing heuristics
+// decide elsewhere.  The hardware compares the per-lane offset with the descriptor's size: a lane whose
+// offset is kLaneOutOfRange reads nothing and receives zeros.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+constexpr uint32_t kLaneOutOfRange = 0x80000000u;
+constexpr int kLoadNonTemporal = 2; // cache-policy bits of the buffer builtins: bit 1 = nt
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void *base)
+{
+    // stride 0 (raw), 2^31 addressable bytes past `base`, 32-bit data format
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)kLaneOutOfRange, 0x00020000);
+}
+
 // RoPE of one interleaved pair; the operation order is part of the contract with the CPU
 // checker so that the appended cache row is bit-identical:
 //   o0 = fma(x0, c, -(x1*s)),  o1 = fma(x1, c, x0*s)      (decoder_kernels.cu:455-458)
@@ -201,12 +216,41 @@ struct CombineShared {
     float4 acc[SG][D / 4];
 };
 
+// Loads and stores of split partials.  DEVICE_COHERENT: relaxed atomic accesses at device scope, which
+// go past the caches that are private to a compute unit or to one of the eight XCDs (each XCD has its own
+// L2), so that a workgroup on one XCD reads what a workgroup on another has written in the same launch
+// — without the whole-cache write-back and invalidation that a device-scope fence costs on this chip.
+template <bool DEVICE_COHERENT>
+__device__ __forceinline__ float load_partial(const float *p)
+{
+    if constexpr (DEVICE_COHERENT) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else return *p;
+}
+
+template <bool DEVICE_COHERENT>
+__device__ __forceinline__ float4 load_partial4(const float4 *p)
+{
+    if constexpr (DEVICE_COHERENT) {
+        const float *f = reinterpret_cast<const float *>(p);
+        return make_float4(load_partial<true>(f), load_partial<true>(f + 1), load_partial<true>(f + 2), load_partial<true>(f + 3));
+    } else {
+        return *p;
+    }
+}
+
+template <bool DEVICE_COHERENT>
+__device__ __forceinline__ void store_partial(float *p, float v)
+{
+    if constexpr (DEVICE_COHERENT) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+
 // Merges the (m, l, o[D]) partials of the first nsp splits of one (b,h), by the 256 threads of a workgroup:
 //   M = max_s m_s;  w_s = exp(m_s - M);  out[d] = sum_s w_s o_s[d] / sum_s w_s l_s.
 // The weights are computed once per split (threads over s), then the weighted sum over splits runs
 // with D/4 threads per split-group (float4 per thread) and 256/(D/4) split-groups side by side, so
 // the partial loads of a group are independent and in flight together.
-template <int D>
+template <int D, bool DEVICE_COHERENT>
 __device__ __forceinline__ void combine_partials(const Params &p, int bh, int nsp, int tid, CombineShared<D> &sh)
 {
     constexpr int TPG = CombineShared<D>::TPG, SG = CombineShared<D>::SG;
@@ -216,7 +260,7 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
 
     float mx = floor_m;
     for (int s = tid; s < nsp; s += kCombineThreads) {
-        const float ms = p.part_m[slot0 + s];
+        const float ms = load_partial<DEVICE_COHERENT>(p.part_m + slot0 + s);
         sh.w[s] = ms;
         mx = fmaxf(mx, ms);
     }
@@ -232,7 +276,7 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
         const float dm = sh.w[s] - M;
         const float w = p.log2_domain ? __builtin_amdgcn_exp2f(dm) : expf(dm);
         sh.w[s] = w;
-        lsum = fmaf(p.part_l[slot0 + s], w, lsum);
+        lsum = fmaf(load_partial<DEVICE_COHERENT>(p.part_l + slot0 + s), w, lsum);
     }
     lsum = wave_sum(lsum);
     if ((tid & 63) == 0) sh.red[1][tid >> 6] = lsum;
@@ -252,7 +296,7 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
 #pragma unroll
         for (int k = 0; k < 4; ++k)
 #pragma unroll
-            for (int v = 0; v < VPT; ++v) x[k][v] = po[(size_t)(s + k * SG) * (D / 4) + v * TPG + t];
+            for (int v = 0; v < VPT; ++v) x[k][v] = load_partial4<DEVICE_COHERENT>(po + (size_t)(s + k * SG) * (D / 4) + v * TPG + t);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const float w = sh.w[s + k * SG];
@@ -269,7 +313,7 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
         const float w = sh.w[s];
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
-            const float4 x = po[(size_t)s * (D / 4) + v * TPG + t];
+            const float4 x = load_partial4<DEVICE_COHERENT>(po + (size_t)s * (D / 4) + v * TPG + t);
             acc[v].x = fmaf(x.x, w, acc[v].x);
             acc[v].y = fmaf(x.y, w, acc[v].y);
             acc[v].z = fmaf(x.z, w, acc[v].z);
@@ -310,7 +354,7 @@ __global__ __launch_bounds__(kCombineThreads) void decode_attn_combine_kernel(co
         for (int d = tid; d < D; d += kCombineThreads) p.out[(size_t)bh * D + d] = __builtin_nanf("");
         return;
     }
-    combine_partials<D>(p, bh, active_splits(p, P), tid, sh);
+    combine_partials<D, false>(p, bh, active_splits(p, P), tid, sh);
 }
 
 // ---------------------------------------------------------------- streaming (split) kernel
@@ -387,41 +431,52 @@ void decode_attn_split_kernel(const Params p)
     const char *Vb = reinterpret_cast<const char *>(p.v_cache) + (size_t)bh * L * ROW_BYTES;
     const uint32_t lane_off = (uint32_t)(group * ROW_BYTES + lig * 16);
     const float *mrow = HAS_MASK ? p.attn_mask + (size_t)P * p.mask_ld : nullptr;
+    // descriptors of this (b,h)'s K rows, V rows and mask row; row offsets go into the scalar offset
+    // (the host checks that L * ROW_BYTES fits 32 bits)
+    const __amdgpu_buffer_rsrc_t Kbuf = make_buffer(Kb), Vbuf = make_buffer(Vb);
+    const __amdgpu_buffer_rsrc_t Mbuf = make_buffer(HAS_MASK ? (const void *)mrow : (const void *)Kb);
 
     // One tile = UNROLL rows per lane-group.  CHECK guards the ragged last tile.
     V kv[UNROLL][CPL], vv[UNROLL][CPL];
-    float mk[UNROLL];
     bool ok[UNROLL];
     constexpr int ROWS_PER_TILE = GROUPS * UNROLL;
+    // Mask entries of a tile: lane-group `group` needs those of rows r0 + u*GROUPS + group, u < UNROLL.
+    // Each lane fetches ONE of them — that of u = lane % 4 — so a single load instruction and a single
+    // register carry the tile's mask, and a quad broadcast (DPP) hands entry u to every lane when the
+    // scores are formed.  (One load per (lane, u) kept four more registers live across the K/V loads,
+    // which the 64-register budget of the 8-waves-per-SIMD occupancy does not have.)
+    static_assert(!HAS_MASK || (LPR >= 4 && UNROLL <= 4), "the mask broadcast works on quads of lanes");
+    float mkv = 0.f;
+    const uint32_t mask_off = (uint32_t)((((lane & 3) < UNROLL ? (lane & 3) : 0) * GROUPS + group) * 4);
 
     // Issues every load of the tile that starts at row r0 and fences the scheduler so that all
     // 2*UNROLL*CPL of them stay in flight together.
     auto issue_tile = [&](int r0, auto check_tag) {
         constexpr bool CHECK = decltype(check_tag)::value;
-        const char *kt = Kb + (size_t)r0 * ROW_BYTES; // uniform
-        const char *vt = Vb + (size_t)r0 * ROW_BYTES;
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            uint32_t off = lane_off + (uint32_t)(u * GROUPS * ROW_BYTES);
-            ok[u] = !CHECK || (r0 + u * GROUPS + group) < cache_end;
-            if (CHECK && !ok[u]) off = (uint32_t)(lig * 16); // row r0: valid; its data is discarded
-#pragma unroll
-            for (int c = 0; c < CPL; ++c)
-                kv[u][c] = __builtin_nontemporal_load(reinterpret_cast<const V *>(kt + off + c * LPR * 16));
-            if constexpr (HAS_MASK) {
-                const int row = (CHECK && !ok[u]) ? r0 : r0 + u * GROUPS + group;
-                mk[u] = mrow[row];
-            } else {
-                mk[u] = 0.f;
-            }
+        const uint32_t tile_off = (uint32_t)r0 * (uint32_t)ROW_BYTES; // uniform
+        if constexpr (HAS_MASK) { // first, so that it has landed when the K rows have
+            uint32_t moff = mask_off;
+            if (CHECK && r0 + (int)(moff >> 2) >= cache_end) moff = kLaneOutOfRange; // reads nothing; the score is discarded
+            mkv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(Mbuf, moff, (uint32_t)r0 * 4u, 0));
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            uint32_t off = lane_off + (uint32_t)(u * GROUPS * ROW_BYTES);
-            if (CHECK && !ok[u]) off = (uint32_t)(lig * 16);
+            ok[u] = !CHECK || (r0 + u * GROUPS + group) < cache_end;
+            const uint32_t off = (CHECK && !ok[u]) ? kLaneOutOfRange : lane_off; // rows past the end: zeros, discarded
 #pragma unroll
             for (int c = 0; c < CPL; ++c)
-                vv[u][c] = __builtin_nontemporal_load(reinterpret_cast<const V *>(vt + off + c * LPR * 16));
+                kv[u][c] = __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(
+                                                     Kbuf, off + (uint32_t)(c * LPR * 16),
+                                                     tile_off + (uint32_t)(u * GROUPS * ROW_BYTES), kLoadNonTemporal));
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint32_t off = (CHECK && !ok[u]) ? kLaneOutOfRange : lane_off;
+#pragma unroll
+            for (int c = 0; c < CPL; ++c)
+                vv[u][c] = __builtin_bit_cast(V, __builtin_amdgcn_raw_buffer_load_b128(
+                                                     Vbuf, off + (uint32_t)(c * LPR * 16),
+                                                     tile_off + (uint32_t)(u * GROUPS * ROW_BYTES), kLoadNonTemporal));
         }
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -471,9 +526,17 @@ void decode_attn_split_kernel(const Params p)
         }
         group_sum_n<LPR, UNROLL>(s);
         float tmax = m;
+        float mk[UNROLL];
+        if constexpr (HAS_MASK) { // entry u of the tile's mask sits in lane u of every quad
+            const float mq = FAST ? mkv * kLog2e : mkv;
+            mk[0] = dpp_move<0x00>(mq);
+            if constexpr (UNROLL > 1) mk[1] = dpp_move<0x55>(mq);
+            if constexpr (UNROLL > 2) mk[2] = dpp_move<0xAA>(mq);
+            if constexpr (UNROLL > 3) mk[3] = dpp_move<0xFF>(mq);
+        }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            s[u] = HAS_MASK ? fmaf(s[u], scale, FAST ? mk[u] * kLog2e : mk[u]) : s[u] * scale;
+            s[u] = HAS_MASK ? fmaf(s[u], scale, mk[u]) : s[u] * scale;
             if (CHECK && !ok[u]) s[u] = -__builtin_inff();
             tmax = fmaxf(tmax, s[u]);
         }
@@ -590,32 +653,32 @@ void decode_attn_split_kernel(const Params p)
             p.out[(size_t)bh * D + d] = O / Lsum; // p = e / sum (decoder_kernels.cu:833)
         } else {
             const size_t slot = (size_t)bh * p.split_cap + split;
-            p.part_o[slot * D + d] = O;
+            store_partial<FUSED>(p.part_o + slot * D + d, O);
             if (d == 0) {
-                p.part_m[slot] = M;
-                p.part_l[slot] = Lsum;
+                store_partial<FUSED>(p.part_m + slot, M);
+                store_partial<FUSED>(p.part_l + slot, Lsum);
             }
         }
     }
 
     if constexpr (FUSED) {
         if (!p.direct) {
-            // Publish the partial device-wide (the other splits of this (b,h) run on other XCDs, each
-            // behind its own L2), count this workgroup in, and let the last one to arrive merge.
-            __threadfence();
+            // The partial went out through device-coherent stores; the barrier waits until every store of
+            // the workgroup has been performed.  Then the workgroup counts itself in, and the last one
+            // to arrive for this (b,h) merges: its device-coherent loads see every partial counted before.
             __syncthreads();
             const int nsp = active_splits(p, P);
             if (tid == 0) {
-                const int before = __hip_atomic_fetch_add(p.arrivals + bh, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+#ifndef FLATTN_ARRIVAL_ORDER
+#define FLATTN_ARRIVAL_ORDER __ATOMIC_RELAXED
+#endif
+                const int before = __hip_atomic_fetch_add(p.arrivals + bh, 1, FLATTN_ARRIVAL_ORDER, __HIP_MEMORY_SCOPE_AGENT);
                 s_last = before == nsp - 1;
                 if (before == nsp - 1) // every split has arrived: nobody touches the counter again in this launch
                     __hip_atomic_store(p.arrivals + bh, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             __syncthreads();
-            if (s_last) {
-                __threadfence(); // partial lines this XCD's caches may still hold from an earlier launch are dropped
-                combine_partials<D>(p, bh, nsp, tid, s_merge);
-            }
+            if (s_last) combine_partials<D, true>(p, bh, nsp, tid, s_merge);
         }
     }
 }
