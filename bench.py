@@ -41,6 +41,8 @@ WORKLOADS = {
     "xb32": dict(B=32, H=32, D=128, ctx=2048, L=2048, dtype="f16", copies=1),
     "xb16": dict(B=16, H=32, D=128, ctx=2048, L=2048, dtype="f16", copies=1),
     "xb4": dict(B=4, H=32, D=128, ctx=2048, L=2048, dtype="f16", copies=4),
+    "xb1_c1024": dict(B=1, H=32, D=128, ctx=1024, L=4096, dtype="f16", copies=12),  # cfg4 with a quarter / half of
+    "xb1_c2048": dict(B=1, H=32, D=128, ctx=2048, L=4096, dtype="f16", copies=12),  # the context: fixed vs per-byte cost
     "xd64": dict(B=64, H=64, D=64, ctx=2048, L=2048, dtype="f16", copies=1),
     "xd256": dict(B=64, H=16, D=256, ctx=2048, L=2048, dtype="f16", copies=1),
 }
@@ -101,12 +103,7 @@ def bench_prefill(args) -> int:
     steps, warm = min(args.steps, 50), min(args.warmup, 5)
     run(warm)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    run(steps)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / steps
+    ms, ms_all = time_region(torch, stream, run, steps, args.repeats)
     dense_flops = 4.0 * B * H * S * (P + S) * D  # every query against every key
     # FLOPs the kernels execute: 32x32 tiles whose mask entries are all <= -1e30 are dropped (their weights
     # are exactly 0); every other tile is multiplied.
@@ -139,7 +136,8 @@ def bench_prefill(args) -> int:
                "gpu_vs_oracle_max_abs_err": max_err}
     print(json.dumps({
         "metric": f"prompt-phase attention TFLOP/s, {args.workload}", "value": round(tflops, 2), "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": round(ms, 5), "higher_is_better": True,
+        "n_gpus": 1, "steps": steps, "warmup": warm, "repeats": args.repeats, "ms_per_step": round(ms, 5),
+        "ms_per_step_all_regions": [round(x, 5) for x in ms_all], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 MFMA, f32 accumulate (f16 storage)" if w["dtype"] == "f16" else "f32 MFMA",
         "data": "synthetic (seeded splitmix64 + Box-Muller N(0,1), seed %d)" % args.seed,
@@ -157,13 +155,20 @@ def bench_prefill(args) -> int:
         "cpu_baseline": cpu}), flush=True)
     return 0
 
-# HBM bytes per launch of the streaming kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
-# scaled by the factor the same counters read for a copy kernel of known size.  Filled in from
-# the summaries under profiles/ (None until measured for that workload).
-MEASURED_TRAFFIC_BYTES = {
-    # profiles/decode_attn_split_kernel_f16_b64_h32_d128_ctx2048.md
-    "cfg3": 2150757750,
-}
+def measured_traffic(workload: str, mask: str):
+    """HBM bytes per launch of the streaming kernel for this workload, as measured with rocprofv3 --pmc
+    (FETCH_SIZE and WRITE_SIZE runs, scaled by what the same counters read for a copy kernel of known
+    size) and recorded in profiles/hbm_traffic_per_launch.md; (None, None) when no row matches."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_per_launch.md")
+    try:
+        with open(path) as f:
+            for line in f:
+                cells = [c.strip() for c in line.strip().strip("|").split("|")]
+                if len(cells) >= 3 and cells[0] == workload and cells[1] == mask and cells[2].isdigit():
+                    return int(cells[2]), "profiles/hbm_traffic_per_launch.md"
+    except OSError:
+        pass
+    return None, None
 
 
 def algorithmic_bytes(B, H, D, e, sum_ctx, has_mask=False, mean_ctx=0):
@@ -176,80 +181,38 @@ def algorithmic_bytes(B, H, D, e, sum_ctx, has_mask=False, mean_ctx=0):
     return kv + tok + out + small
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS) + sorted(PREFILL_WORKLOADS) + ["all"],
-                    help="'all' prints one JSON line per configuration cfg1..cfg5 (each in a child process)")
-    ap.add_argument("--nsplit", type=int, default=0, help="force the context split count (0 = library's choice)")
-    ap.add_argument("--seed", type=int, default=1234)
-    ap.add_argument("--graph-steps", type=int, default=20,
-                    help="also time the step replayed from a HIP graph of this many steps (0 = skip)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--calib-copy", action="store_true",
-                    help="only run a plain 1 GiB -> 1 GiB elementwise copy kernel a few times (for scaling "
-                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings), then exit")
-    ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
-    ap.add_argument("--prefill-mask", default="causal", choices=["causal", "causal-1e5", "block-causal", "none"],
-                    help="prompt-phase workloads: additive causal mask with -FLT_MAX (the reference's driver) or "
-                         "-1e5 (its kernel harness) above the diagonal, or no mask")
-    ap.add_argument("--prefill-fast-qk", action="store_true",
-                    help="prompt-phase fp16 workloads: FL_ATTN_FLAG_FAST_PROMPT_QK (queries as one fp16 value)")
-    ap.add_argument("--mask", default="none", choices=["none", "causal", "strict"],
-                    help="decode workloads: additive mask [L, L] with row stride L, row start_pos is used "
-                         "(open_decoder.cu:207): causal = 0 up to and including the new token, -FLT_MAX beyond; "
-                         "strict = the reference driver's mask, which also hides the new token "
-                         "(samples/llama_fp16.cu:73-81)")
-    ap.add_argument("--two-launches", action="store_true",
-                    help="decode workloads: skip fl_decode_attn_workspace_init, so that a split context is merged "
-                         "by a second launch instead of inside the streaming kernel")
-    ap.add_argument("--segment", default="attention", choices=["attention", "int32-int8"],
-                    help="attention: q/k/v in the cache dtype -> float output (the headline metric). "
-                         "int32-int8: the whole reference segment, int32 GEMM accumulators + scales in, "
-                         "per-token INT8 + scale out (implies --no-cpu)")
-    args = ap.parse_args()
+def median(xs):
+    xs = sorted(xs)
+    n = len(xs)
+    return xs[n // 2] if n % 2 else 0.5 * (xs[n // 2 - 1] + xs[n // 2])
 
-    if args.workload == "all":
-        import subprocess
-        rc = 0
-        for w in ("cfg1", "cfg2", "cfg3", "cfg4", "cfg5"):
-            cmd = [sys.executable, os.path.abspath(__file__), "--workload", w, "--steps", str(args.steps),
-                   "--warmup", str(args.warmup), "--seed", str(args.seed)] + (["--no-cpu"] if args.no_cpu else [])
-            rc |= subprocess.run(cmd).returncode
-        return rc
 
-    if args.workload in PREFILL_WORKLOADS and args.gpus == 1:
-        return bench_prefill(args)
+def time_region(torch, stream, run, steps, repeats):
+    """ms per step of `run(steps)` between two events on `stream`: the median of `repeats` timed regions
+    (and every region's figure)."""
+    per_step = []
+    for _ in range(repeats):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        run(steps)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        per_step.append(e0.elapsed_time(e1) / steps)
+    return median(per_step), per_step
 
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (the path has no cross-GPU exchange); "
-              "run with --gpus 1", file=sys.stderr)
-        return 2
 
+def measure_decode(name, args, steps, warmup, repeats, mask="none", graph_steps=0, cpu=False, two_launches=False,
+                   segment="attention", nsplit=0):
+    """One decode workload: inputs to HBM, timed regions of the whole step and of the streaming kernel
+    alone, optionally the HIP-graph replay and the CPU baseline.  Returns a dict of plain numbers."""
     import numpy as np
     import torch
 
     from fasterllama_amd import capi, synth
     from fasterllama_amd.decode_attn import DecodeAttention
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        return 3
-    capi.load()  # fails loudly when the HIP library is missing
     dev = torch.device("cuda:0")
-    if args.calib_copy:
-        n = 1 << 28  # 2^28 floats = 1 GiB read + 1 GiB written per launch
-        src = torch.ones(n, dtype=torch.float32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            torch.mul(src, 1.0, out=dst)
-        torch.cuda.synchronize()
-        print(json.dumps({"calib_copy": True, "bytes_read_per_launch": n * 4, "bytes_written_per_launch": n * 4,
-                          "launches": 5}), flush=True)
-        return 0
-    w = WORKLOADS[args.workload]
+    w = WORKLOADS[name]
     B, H, D, L = w["B"], w["H"], w["D"], w["L"]
     np_dt = np.float16 if w["dtype"] == "f16" else np.float32
     t_dt = torch.float16 if w["dtype"] == "f16" else torch.float32
@@ -282,29 +245,26 @@ def main() -> int:
     q, k, v = (torch.from_numpy(a).to(dev) for a in (q_h, k_h, v_h))
     freq = torch.from_numpy(freq_h).to(dev)
     mask_h = None
-    if args.mask != "none":
+    if mask != "none":
         fmax = float(np.finfo(np.float32).max)
         r, c = np.arange(L)[:, None], np.arange(L)[None, :]
-        mask_h = np.where(c <= r if args.mask == "causal" else c < r, 0.0, -fmax).astype(np.float32)
+        mask_h = np.where(c <= r if mask == "causal" else c < r, 0.0, -fmax).astype(np.float32)
     mask_d = None if mask_h is None else torch.from_numpy(mask_h).to(dev)
     pos_d = torch.from_numpy(pos_h).to(dev) if ragged else None
     # small workloads rotate over several cache copies so the rows do not sit in the 256 MB MALL
-    caches = []
-    for c in range(copies):
-        caches.append((torch.from_numpy(kc_h).to(dev), torch.from_numpy(vc_h).to(dev)))
+    caches = [(torch.from_numpy(kc_h).to(dev), torch.from_numpy(vc_h).to(dev)) for _ in range(copies)]
     out = torch.empty(B, H * D, dtype=torch.float32, device=dev)
     torch.cuda.synchronize()
     gen_s = time.time() - t0
 
-    op = DecodeAttention(B, H, D, L, t_dt, nsplit=args.nsplit, device=dev)
-    if not args.two_launches:
-        op.init_workspace()  # split steps run as one launch (the last workgroup of each (b,h) merges)
+    op = DecodeAttention(B, H, D, L, t_dt, nsplit=nsplit, device=dev)
+    if not two_launches:
+        op.init_workspace()  # a split context is merged inside the streaming kernel: one launch per step
     plan = op.plan(max_ctx, ragged)
     extra = {}
-    if args.segment == "int32-int8":
+    if segment == "int32-int8":
         # the segment as OpenDecoder::forward feeds it: int32 accumulators of the INT8 projections with
         # activation/weight scales in, quantised attention output out
-        args.no_cpu = True
         rng = np.random.default_rng(args.seed)
         q, k, v = (torch.from_numpy(rng.integers(-20000, 20000, (B, 1, H, D), dtype=np.int32)).to(dev)
                    for _ in range(3))
@@ -325,34 +285,31 @@ def main() -> int:
             if st != 0:
                 raise capi.FlAttnError(st, capi.strerror(st))
 
-    # ---- timed region: W warm-up steps, then exactly K steps between two events on the stream
-    run(args.warmup)
+    # ---- timed regions: W warm-up steps, then `repeats` regions of exactly K steps each between two
+    # events on the launch stream; the median region is reported
+    run(warmup)
     torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     h0 = time.perf_counter()
-    ev0.record(stream)
-    run(args.steps)
-    ev1.record(stream)
-    torch.cuda.synchronize()
+    step_ms, step_all = time_region(torch, stream, run, steps, repeats)
     host_ms = (time.perf_counter() - h0) * 1e3
-    step_ms = ev0.elapsed_time(ev1) / args.steps
     out_gpu = out.cpu().numpy().copy()
 
-    # ---- the streaming kernel alone (pass 1), same launches, same stream
-    run(max(3, args.warmup // 4), passes=1)
-    torch.cuda.synchronize()
-    ev2, ev3 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    ev2.record(stream)
-    run(args.steps, passes=1)
-    ev3.record(stream)
-    torch.cuda.synchronize()
-    kern_ms = ev2.elapsed_time(ev3) / args.steps
+    # ---- the streaming kernel alone (pass 1), same launches, same stream.  When the step is one launch
+    # (no split, or a split merged inside the kernel) that launch IS the step.
+    launches = 1 if plan.two_pass == 0 or (plan.two_pass == 2 and not two_launches) else 2
+    one_launch = launches == 1 and segment == "attention"
+    if one_launch:
+        kern_ms, kern_all = step_ms, step_all
+    else:
+        run(max(3, warmup // 4), passes=1)
+        torch.cuda.synchronize()
+        kern_ms, kern_all = time_region(torch, stream, lambda n: run(n, passes=1), steps, repeats)
 
     # ---- the same step replayed from a HIP graph (how a serving loop hides launch gaps): G steps per
     # graph, rotating over the cache copies like the eager loop; reported beside the eager figure
     graph_us = None
-    if args.graph_steps > 0:
-        G = max(copies, args.graph_steps // copies * copies)
+    if graph_steps > 0:
+        G = max(copies, graph_steps // copies * copies)
         side = torch.cuda.Stream(device=dev)
         g = torch.cuda.CUDAGraph()
         with torch.cuda.stream(side):
@@ -363,60 +320,243 @@ def main() -> int:
                     if st != 0:
                         raise capi.FlAttnError(st, capi.strerror(st))
         torch.cuda.synchronize()
-        reps = max(1, args.steps // G)
+        reps = max(1, steps // G)
         for _ in range(2):
             g.replay()
         torch.cuda.synchronize()
-        ev4, ev5 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        ev4.record(stream)
-        for _ in range(reps):
-            g.replay()
-        ev5.record(stream)
-        torch.cuda.synchronize()
-        graph_us = ev4.elapsed_time(ev5) / (reps * G) * 1e3
+        graph_ms, _ = time_region(torch, stream, lambda n: [g.replay() for _ in range(n)], reps, repeats)
+        graph_us = graph_ms / G * 1e3
         if not np.array_equal(out.cpu().numpy(), out_gpu):
             raise RuntimeError("HIP-graph replay and eager step disagree")
 
     alg = algorithmic_bytes(B, H, D, e, sum_ctx, has_mask=mask_h is not None, mean_ctx=sum_ctx / B)
-    gbps = alg / (step_ms * 1e-3) / 1e9
-    kern_gbps = alg / (kern_ms * 1e-3) / 1e9
+    res = dict(
+        name=name, B=B, H=H, D=D, L=L, dtype=w["dtype"], ragged=ragged, mask=mask, copies=copies, sum_ctx=sum_ctx,
+        max_ctx=max_ctx, nsplit=plan.nsplit, chunk_rows=plan.chunk_rows,
+        launches_per_step=launches + (1 if segment == "int32-int8" else 0),
+        alg_bytes=alg, step_ms=step_ms, step_ms_all=step_all, kern_ms=kern_ms, kern_ms_all=kern_all,
+        graph_us=graph_us, host_ms=host_ms, gen_s=gen_s, cpu=None)
 
-    # ---- CPU baseline: the scalar oracle on a bounded sample of the same inputs (~10-20 s of CPU work)
-    cpu = None
-    max_err = None
-    if not args.no_cpu:
+    # ---- CPU baseline: the scalar oracle on the same inputs.  The full batch when one single-thread pass
+    # stays within a few seconds (the headline does: ~1.2 s), else the leading sequences.
+    if cpu:
         from oracle import ref  # checker / baseline only
         per_seq = 2 * H * D * e * (sum_ctx / B)
-        ns = args.cpu_seqs or max(1, min(B, int(round(0.5e9 / per_seq))))  # ~0.5 GB of K+V per pass
+        ns = args.cpu_seqs or max(1, min(B, int(round(2.2e9 / per_seq))))
         sl = slice(0, ns)
         pos_s = pos_h[sl] if ragged else None
         sample_bytes = algorithmic_bytes(ns, H, D, e, int(lens[sl].sum()), has_mask=mask_h is not None,
                                          mean_ctx=float(lens[sl].mean()))
 
-        def cpu_leg(threads, budget_s, max_reps):
+        def cpu_leg(threads, budget_s, min_reps, max_reps):
             kc_s, vc_s = kc_h[sl].copy(), vc_h[sl].copy()
-            times, res = [], None
-            while sum(times) < budget_s and len(times) < max_reps:
+            times, r = [], None
+            while len(times) < min_reps or (sum(times) < budget_s and len(times) < max_reps):
                 t1 = time.perf_counter()
-                res = ref.decode_attn(q_h[sl], k_h[sl], v_h[sl], kc_s, vc_s, freq_h, start_pos=start_pos,
-                                      start_pos_per_seq=pos_s, attn_mask=mask_h, threads=threads)
+                r = ref.decode_attn(q_h[sl], k_h[sl], v_h[sl], kc_s, vc_s, freq_h, start_pos=start_pos,
+                                    start_pos_per_seq=pos_s, attn_mask=mask_h, threads=threads)
                 times.append(time.perf_counter() - t1)
-            return res, min(times), len(times), sum(times)
+            return r, median(times), len(times), sum(times)
 
-        out_ref, cpu_1t, reps_1t, total_1t = cpu_leg(1, 10.0, 50)
+        out_ref, cpu_1t, reps_1t, total_1t = cpu_leg(1, 8.0, 3, 50)
         nthreads = max(1, min(16, os.cpu_count() or 1))
-        _, cpu_nt, reps_nt, total_nt = cpu_leg(nthreads, 4.0, 50)
-        max_err = float(np.abs(out_gpu[sl] - out_ref).max())
-        cpu = {
+        _, cpu_nt, reps_nt, total_nt = cpu_leg(nthreads, 4.0, 3, 50)
+        res["cpu"] = {
             "value": round(sample_bytes / cpu_1t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"first {ns} of {B} sequences of the same seeded inputs ({sample_bytes / 1e6:.0f} MB "
-                      f"algorithmic per pass), scalar oracle, 1 thread, best of {reps_1t} passes "
-                      f"({total_1t:.1f} s of CPU work)",
-            "us_per_step_scaled_to_full_batch": round(cpu_1t * B / ns * 1e6, 1),
+            "sample": (f"all {B} sequences" if ns == B else f"first {ns} of {B} sequences") +
+                      f" of the same seeded inputs ({sample_bytes / 1e6:.0f} MB algorithmic per pass), scalar oracle, "
+                      f"1 thread, median of {reps_1t} passes ({total_1t:.1f} s of CPU work)",
+            "us_per_step": round(cpu_1t * B / ns * 1e6, 1),
             "openmp": {"value": round(sample_bytes / cpu_nt / 1e9, 4), "unit": "GB/s", "cores": nthreads,
-                       "passes": reps_nt, "us_per_step_scaled_to_full_batch": round(cpu_nt * B / ns * 1e6, 1)},
-            "gpu_vs_oracle_max_abs_err": max_err,
+                       "passes": reps_nt, "us_per_step": round(cpu_nt * B / ns * 1e6, 1)},
+            "gpu_vs_oracle_max_abs_err": float(np.abs(out_gpu[sl] - out_ref).max()),
         }
+    del caches, ios, op
+    torch.cuda.empty_cache()
+    return res
+
+
+def summary(res):
+    """The figures of one workload as they appear under other_configs."""
+    gbps = res["alg_bytes"] / (res["step_ms"] * 1e-3) / 1e9
+    return {
+        "workload": describe(res), "us_per_step": round(res["step_ms"] * 1e3, 2), "GBps": round(gbps, 1),
+        "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "nsplit": res["nsplit"],
+        "launches_per_step": res["launches_per_step"], "algorithmic_bytes_per_step": res["alg_bytes"],
+        "us_per_step_all_regions": [round(x * 1e3, 2) for x in res["step_ms_all"]],
+    }
+
+
+def describe(res):
+    return (f"{res['name']}: decode self-attention step, B={res['B']} H={res['H']} D={res['D']} "
+            + (f"ragged ctx U[1,{res['L']}] (sum {res['sum_ctx']})" if res["ragged"] else f"ctx={res['max_ctx']}")
+            + f" L={res['L']} {res['dtype']} KV cache, RoPE at position, "
+            + {"none": "no mask", "causal": "causal additive mask row (0 / -FLT_MAX)",
+               "strict": "the reference driver's strict mask row (new token hidden)"}[res["mask"]])
+
+
+def calibrate(args) -> int:
+    """Measurement-only legs: what the memory system, the matrix cores and the launch path of this
+    machine sustain (kernels of libfl_calib.so, none of them part of the attention path)."""
+    import ctypes as C
+
+    import torch
+
+    from fasterllama_amd import build
+    if build.is_stale("calib"):
+        build.build_calib()
+    lib = C.CDLL(build.outputs("calib"))
+    lib.fl_calib_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    lib.fl_calib_mfma.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    lib.fl_calib_empty.argtypes = [C.c_void_p]
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream(dev)
+    sp = C.c_void_p(stream.cuda_stream)
+    sink = torch.zeros(4, dtype=torch.float32, device=dev)
+
+    def timed(fn, n):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        ms, _ = time_region(torch, stream, lambda k: [fn() for _ in range(k)], n, 5)
+        return ms
+
+    def ok(rc):
+        if rc != 0:
+            raise RuntimeError(f"calibration launch failed: hipError {rc}")
+
+    out = {"calib": args.calib}
+    if args.calib == "copy":
+        n = 1 << 28  # 2^28 floats = 1 GiB read + 1 GiB written per launch
+        src = torch.ones(n, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        out.update(bytes_read_per_launch=n * 4, bytes_written_per_launch=n * 4, launches=5)
+    elif args.calib == "read":
+        nbytes = 2 << 30  # the headline step reads 2 GiB of K and V
+        buf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        buf.random_(0, 256)
+        rows = []
+        for blocks in (256, 512, 2048, 8192):
+            for nt in (0, 1):
+                ms = timed(lambda: ok(lib.fl_calib_stream_read(buf.data_ptr(), nbytes, blocks, nt, sink.data_ptr(), sp)), 20)
+                rows.append({"workgroups": blocks, "loads": "nt" if nt else "plain", "us": round(ms * 1e3, 1),
+                             "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)})
+        out.update(bytes=nbytes, pattern="128-bit loads, 8 per lane in flight, one contiguous slice per workgroup", results=rows)
+    elif args.calib == "mfma":
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        rows = []
+        for fp32, iters, flop in ((0, 20000, 2 * 32 * 32 * 16), (1, 20000, 2 * 32 * 32 * 2)):
+            for wgs_per_cu in (1, 2):
+                for rnd in (0, 1):
+                    blocks = cus * wgs_per_cu
+                    ms = timed(lambda: ok(lib.fl_calib_mfma(fp32, blocks, iters, rnd, sink.data_ptr(), sp)), 5)
+                    flops = blocks * 4 * 4 * iters * flop
+                    rows.append({"mfma": "v_mfma_f32_32x32x2_f32" if fp32 else "v_mfma_f32_32x32x16_f16",
+                                 "waves_per_simd": wgs_per_cu, "operands": "random in [-2,2]" if rnd else "zeros",
+                                 "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1)})
+        out.update(compute_units=cus, results=rows)
+    elif args.calib == "launch":
+        ms = timed(lambda: ok(lib.fl_calib_empty(sp)), 2000)
+        out.update(empty_kernel_us_per_launch=round(ms * 1e3, 3),
+                   note="back-to-back launches of an empty kernel on one stream, HIP events around 2000 of them")
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="timed regions of --steps steps each; the median region is reported")
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS) + sorted(PREFILL_WORKLOADS) + ["all"],
+                    help="'all' prints one JSON line per configuration cfg1..cfg5 (each in a child process)")
+    ap.add_argument("--nsplit", type=int, default=0, help="force the context split count (0 = library's choice)")
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--graph-steps", type=int, default=20,
+                    help="also time the step replayed from a HIP graph of this many steps (0 = skip)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-others", action="store_true",
+                    help="skip the other_configs object (the remaining configurations, measured in the same run "
+                         "with the headline workload)")
+    ap.add_argument("--calib", choices=["copy", "read", "mfma", "launch"],
+                    help="measurement-only legs, then exit.  copy: a plain 1 GiB -> 1 GiB elementwise copy (for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings); read: 2 GiB streaming read, plain and non-temporal "
+                         "loads; mfma: register-only MFMA loops; launch: empty-kernel launch cadence")
+    ap.add_argument("--calib-copy", action="store_true", help="same as --calib copy")
+    ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
+    ap.add_argument("--prefill-mask", default="causal", choices=["causal", "causal-1e5", "block-causal", "none"],
+                    help="prompt-phase workloads: additive causal mask with -FLT_MAX (the reference's driver) or "
+                         "-1e5 (its kernel harness) above the diagonal, or no mask")
+    ap.add_argument("--prefill-fast-qk", action="store_true",
+                    help="prompt-phase fp16 workloads: FL_ATTN_FLAG_FAST_PROMPT_QK (queries as one fp16 value)")
+    ap.add_argument("--mask", default="none", choices=["none", "causal", "strict"],
+                    help="decode workloads: additive mask [L, L] with row stride L, row start_pos is used "
+                         "(open_decoder.cu:207): causal = 0 up to and including the new token, -FLT_MAX beyond; "
+                         "strict = the reference driver's mask, which also hides the new token "
+                         "(samples/llama_fp16.cu:73-81)")
+    ap.add_argument("--two-launches", action="store_true",
+                    help="decode workloads: skip fl_decode_attn_workspace_init, so that a split context is merged "
+                         "by a second launch instead of inside the streaming kernel")
+    ap.add_argument("--segment", default="attention", choices=["attention", "int32-int8"],
+                    help="attention: q/k/v in the cache dtype -> float output (the headline metric). "
+                         "int32-int8: the whole reference segment, int32 GEMM accumulators + scales in, "
+                         "per-token INT8 + scale out (implies --no-cpu)")
+    args = ap.parse_args()
+    if args.calib_copy:
+        args.calib = "copy"
+    if args.repeats < 1 or args.steps < 1:
+        ap.error("--steps and --repeats must be positive")
+
+    if args.workload == "all":
+        import subprocess
+        rc = 0
+        for w in ("cfg1", "cfg2", "cfg3", "cfg4", "cfg5"):
+            cmd = [sys.executable, os.path.abspath(__file__), "--workload", w, "--steps", str(args.steps),
+                   "--warmup", str(args.warmup), "--seed", str(args.seed), "--no-others"] + (["--no-cpu"] if args.no_cpu else [])
+            rc |= subprocess.run(cmd).returncode
+        return rc
+
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path has no cross-GPU exchange); "
+              "run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from fasterllama_amd import capi
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    if args.calib:
+        return calibrate(args)
+    if args.workload in PREFILL_WORKLOADS:
+        return bench_prefill(args)
+    capi.load()  # fails loudly when the HIP library is missing
+
+    if args.segment == "int32-int8":
+        args.no_cpu = True
+    res = measure_decode(args.workload, args, args.steps, args.warmup, args.repeats, mask=args.mask,
+                         graph_steps=args.graph_steps, cpu=not args.no_cpu, two_launches=args.two_launches,
+                         segment=args.segment, nsplit=args.nsplit)
+    gbps = res["alg_bytes"] / (res["step_ms"] * 1e-3) / 1e9
+    kern_gbps = res["alg_bytes"] / (res["kern_ms"] * 1e-3) / 1e9
+    traffic, traffic_src = measured_traffic(args.workload, args.mask)
+
+    # ---- the other configurations and the masked headline, measured in the same run (shorter regions)
+    others = None
+    if args.workload == HEADLINE and not args.no_others and args.mask == "none" and args.segment == "attention":
+        others = {}
+        o_steps, o_rep = max(10, min(args.steps, 50)), max(3, min(args.repeats, 3))
+        for key, name, mask in (("cfg1", "cfg1", "none"), ("cfg2", "cfg2", "none"), ("cfg4", "cfg4", "none"),
+                                ("cfg5", "cfg5", "none"), ("cfg3_causal_mask", "cfg3", "causal"),
+                                ("cfg3_strict_mask", "cfg3", "strict")):
+            others[key] = summary(measure_decode(name, args, o_steps, max(3, args.warmup // 2), o_rep, mask=mask))
 
     line = {
         "metric": "decode-attn us/step + HBM GB/s (% peak), LLaMA2-7B heads b=64 ctx=2048 fp16"
@@ -426,37 +566,36 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(step_ms, 6),
-        "us_per_step": round(step_ms * 1e3, 2),
+        "repeats": args.repeats,
+        "ms_per_step": round(res["step_ms"], 6),
+        "us_per_step": round(res["step_ms"] * 1e3, 2),
+        "us_per_step_all_regions": [round(x * 1e3, 2) for x in res["step_ms_all"]],
         "pct_of_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBPS, 2),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16 storage / f32 accumulate" if w["dtype"] == "f16" else "f32",
+        "dtype": "f16 storage / f32 accumulate" if res["dtype"] == "f16" else "f32",
         "data": "synthetic (seeded splitmix64 + Box-Muller N(0,1), seed %d)" % args.seed,
         "config": {
-            "workload": f"{args.workload}: decode self-attention step, B={B} H={H} D={D} "
-                        + (f"ragged ctx U[1,{L}] (sum {sum_ctx})" if ragged else f"ctx={max_ctx}")
-                        + f" L={L} {w['dtype']} KV cache, RoPE at position, "
-                        + {"none": "no mask", "causal": "causal additive mask row (0 / -FLT_MAX)",
-                           "strict": "the reference driver's strict mask row (new token hidden)"}[args.mask],
-            "batch": B, "heads": H, "head_dim": D, "ctx": max_ctx if not ragged else None,
-            "sum_ctx": sum_ctx, "cache_rows": L, "cache_copies_rotated": copies,
-            "nsplit": plan.nsplit, "chunk_rows": plan.chunk_rows,
-            "launches_per_step": 2 if (plan.two_pass and args.two_launches) else 1,
-            "algorithmic_bytes_per_step": alg,
+            "workload": describe(res),
+            "batch": res["B"], "heads": res["H"], "head_dim": res["D"], "ctx": res["max_ctx"] if not res["ragged"] else None,
+            "sum_ctx": res["sum_ctx"], "cache_rows": res["L"], "cache_copies_rotated": res["copies"],
+            "nsplit": res["nsplit"], "chunk_rows": res["chunk_rows"], "launches_per_step": res["launches_per_step"],
+            "algorithmic_bytes_per_step": res["alg_bytes"],
             "segment": args.segment,
+            "timing": f"median of {args.repeats} regions of {args.steps} steps after {args.warmup} warm-up steps, HIP events on the launch stream",
         },
         "roofline": {
             "bound": "hbm", "achieved": round(kern_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(kern_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-            "kernel": "decode_attn_split_kernel", "kernel_us": round(kern_ms * 1e3, 2),
+            "traffic": traffic, "traffic_source": traffic_src,
+            "kernel": "decode_attn_split_kernel", "kernel_us": round(res["kern_ms"] * 1e3, 2),
         },
-        "cpu_baseline": cpu,
-        "hip_graph_us_per_step": None if graph_us is None else round(graph_us, 2),
-        "host_ms_total": round(host_ms, 3),
-        "input_gen_s": round(gen_s, 2),
+        "cpu_baseline": res["cpu"],
+        "other_configs": others,
+        "hip_graph_us_per_step": None if res["graph_us"] is None else round(res["graph_us"], 2),
+        "host_ms_total": round(res["host_ms"], 3),
+        "input_gen_s": round(res["gen_s"], 2),
     }
     print(json.dumps(line), flush=True)
     return 0

@@ -7,8 +7,10 @@ Targets
     hip     fasterllama_amd/lib/libfl_decode_attn.so   HIP kernels + C ABI (include/fl_decode_attn.h)
     cxx     fasterllama_amd/lib/libflopendecoder.so    C++ OpenDecoder mirror over the C ABI
     synth   fasterllama_amd/lib/libfl_synth.so         host-side seeded input generator
+    calib   fasterllama_amd/lib/libfl_calib.so         measurement-only kernels of bench.py --calib
     oracle  oracle/libfl_ref.so                        CPU checker (test infrastructure)
     cpptest tests/cpp/open_decoder_check               C++ drop-in test driver
+    sanitize (by name only) oracle + C-ABI host logic built with ASan/UBSan and run on the CPU
 """
 from __future__ import annotations
 
@@ -34,13 +36,14 @@ HIP_FLAGS = [
 def sources(name: str) -> list[str]:
     """Files a target is built from (a change in any of them makes the built file stale)."""
     import glob
-    hip = sorted(glob.glob(os.path.join(CSRC, "*.hip")) + glob.glob(os.path.join(CSRC, "*.hpp"))) + \
+    hip = [os.path.join(CSRC, "fl_decode_attn.hip")] + sorted(glob.glob(os.path.join(CSRC, "*.hpp"))) + \
         [os.path.join(ROOT, "include", "fl_decode_attn.h")]
     return {
         "hip": hip,
         "cxx": [os.path.join(CSRC, "open_decoder.cpp"), os.path.join(CSRC, "open_decoder.h"),
                 os.path.join(ROOT, "include", "fl_decode_attn.h")],
         "synth": [os.path.join(CSRC, "fl_synth.c")],
+        "calib": [os.path.join(CSRC, "fl_calib.hip")],
         "oracle": [os.path.join(ROOT, "oracle", "fl_ref_decode_attn.c"), os.path.join(ROOT, "oracle", "Makefile")],
         "cpptest": [os.path.join(ROOT, "tests", "cpp", "open_decoder_check.cpp"), os.path.join(CSRC, "open_decoder.h"),
                     os.path.join(ROOT, "include", "fl_decode_attn.h")],
@@ -52,6 +55,7 @@ def outputs(name: str) -> str:
         "hip": os.path.join(LIB, "libfl_decode_attn.so"),
         "cxx": os.path.join(LIB, "libflopendecoder.so"),
         "synth": os.path.join(LIB, "libfl_synth.so"),
+        "calib": os.path.join(LIB, "libfl_calib.so"),
         "oracle": os.path.join(ROOT, "oracle", "libfl_ref.so"),
         "cpptest": os.path.join(ROOT, "tests", "cpp", "open_decoder_check"),
     }[name]
@@ -131,6 +135,14 @@ def build_synth() -> str:
     return _built("synth")
 
 
+def build_calib() -> str:
+    """Measurement-only kernels for bench.py --calib (a library of its own, not linked into the product)."""
+    os.makedirs(LIB, exist_ok=True)
+    out = os.path.join(LIB, "libfl_calib.so")
+    _run([hipcc(), *HIP_FLAGS, "-shared", "-o", out, os.path.join(CSRC, "fl_calib.hip")])
+    return _built("calib")
+
+
 def build_oracle() -> str:
     _run(["make", "-C", os.path.join(ROOT, "oracle"), "-B"])
     return _built("oracle")
@@ -148,17 +160,36 @@ def build_cpptest() -> str:
     return _built("cpptest")
 
 
+def run_sanitizers() -> None:
+    """Host code under AddressSanitizer + UndefinedBehaviorSanitizer, built and RUN here (no GPU involved):
+    the CPU oracle with its driver (`make -C oracle asan`), and the host pass of the C-ABI library with
+    tests/cpp/capi_host_check.cpp (validation, planning and workspace arithmetic; every call is rejected
+    before a launch).  Raises when a sanitizer reports or a check fails."""
+    _run(["make", "-C", os.path.join(ROOT, "oracle"), "-B", "asan"])
+    exe = os.path.join(ROOT, "tests", "cpp", "capi_host_check")
+    _run([hipcc(), f"--offload-arch={GFX_ARCH}", "-O1", "-g", "-std=c++17",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unknown-warning-option",
+          "-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+          "-Xarch_host", "-fno-sanitize-recover=all",
+          "-I", os.path.join(ROOT, "include"), "-o", exe,
+          os.path.join(CSRC, "fl_decode_attn.hip"), os.path.join(ROOT, "tests", "cpp", "capi_host_check.cpp")])
+    _run([exe])
+
+
 TARGETS = {
     "hip": build_hip,
     "cxx": build_cxx,
     "synth": build_synth,
+    "calib": build_calib,
     "oracle": build_oracle,
     "cpptest": build_cpptest,
+    "sanitize": run_sanitizers,
 }
+DEFAULT_TARGETS = [t for t in TARGETS if t != "sanitize"]  # the sanitizer run is asked for by name (and by the CPU tests)
 
 
 def build_all(targets: list[str] | None = None) -> None:
-    for name in targets or list(TARGETS):
+    for name in targets or DEFAULT_TARGETS:
         if name == "cxx" and not os.path.exists(os.path.join(CSRC, "open_decoder.cpp")):
             continue
         if name == "cpptest" and not os.path.exists(os.path.join(ROOT, "tests", "cpp", "open_decoder_check.cpp")):

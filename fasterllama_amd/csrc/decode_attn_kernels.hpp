@@ -258,8 +258,27 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
     const size_t slot0 = (size_t)bh * p.split_cap;
     const float floor_m = p.log2_domain ? kMaxFloor * kLog2e : kMaxFloor;
 
+    // Every load whose address is known up front is issued before the first barrier — the statistics of
+    // the first 256 splits and the first four partial rows of this thread's split-group — so that the
+    // merge waits for memory once, not once per phase.  The arithmetic and its order do not depend on it.
+    const int sg = tid / TPG, t = tid % TPG;
+    const float4 *po = reinterpret_cast<const float4 *>(p.part_o + slot0 * D);
+    const float m_first = tid < nsp ? load_partial<DEVICE_COHERENT>(p.part_m + slot0 + tid) : floor_m;
+    const float l_first = tid < nsp ? load_partial<DEVICE_COHERENT>(p.part_l + slot0 + tid) : 0.f;
+    float4 x_first[4][VPT];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+            x_first[k][v] = sg + k * SG < nsp ? load_partial4<DEVICE_COHERENT>(po + (size_t)(sg + k * SG) * (D / 4) + v * TPG + t)
+                                              : make_float4(0.f, 0.f, 0.f, 0.f);
+
     float mx = floor_m;
-    for (int s = tid; s < nsp; s += kCombineThreads) {
+    if (tid < nsp) {
+        sh.w[tid] = m_first;
+        mx = fmaxf(mx, m_first);
+    }
+    for (int s = tid + kCombineThreads; s < nsp; s += kCombineThreads) {
         const float ms = load_partial<DEVICE_COHERENT>(p.part_m + slot0 + s);
         sh.w[s] = ms;
         mx = fmaxf(mx, ms);
@@ -276,7 +295,7 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
         const float dm = sh.w[s] - M;
         const float w = p.log2_domain ? __builtin_amdgcn_exp2f(dm) : expf(dm);
         sh.w[s] = w;
-        lsum = fmaf(load_partial<DEVICE_COHERENT>(p.part_l + slot0 + s), w, lsum);
+        lsum = fmaf(s == tid ? l_first : load_partial<DEVICE_COHERENT>(p.part_l + slot0 + s), w, lsum);
     }
     lsum = wave_sum(lsum);
     if ((tid & 63) == 0) sh.red[1][tid >> 6] = lsum;
@@ -285,12 +304,22 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
 #pragma unroll
     for (int w = 1; w < kCombineThreads / 64; ++w) Lsum += sh.red[1][w];
 
-    const int sg = tid / TPG, t = tid % TPG;
     float4 acc[VPT];
 #pragma unroll
     for (int v = 0; v < VPT; ++v) acc[v] = make_float4(0.f, 0.f, 0.f, 0.f);
-    const float4 *po = reinterpret_cast<const float4 *>(p.part_o + slot0 * D);
-    int s = sg;
+    auto add_row = [&](const float4 (&x)[VPT], float w) {
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            acc[v].x = fmaf(x[v].x, w, acc[v].x);
+            acc[v].y = fmaf(x[v].y, w, acc[v].y);
+            acc[v].z = fmaf(x[v].z, w, acc[v].z);
+            acc[v].w = fmaf(x[v].w, w, acc[v].w);
+        }
+    };
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        if (sg + k * SG < nsp) add_row(x_first[k], sh.w[sg + k * SG]);
+    int s = sg + 4 * SG;
     for (; s + 3 * SG < nsp; s += 4 * SG) { // four independent partial rows in flight
         float4 x[4][VPT];
 #pragma unroll
@@ -298,27 +327,13 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
 #pragma unroll
             for (int v = 0; v < VPT; ++v) x[k][v] = load_partial4<DEVICE_COHERENT>(po + (size_t)(s + k * SG) * (D / 4) + v * TPG + t);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const float w = sh.w[s + k * SG];
-#pragma unroll
-            for (int v = 0; v < VPT; ++v) {
-                acc[v].x = fmaf(x[k][v].x, w, acc[v].x);
-                acc[v].y = fmaf(x[k][v].y, w, acc[v].y);
-                acc[v].z = fmaf(x[k][v].z, w, acc[v].z);
-                acc[v].w = fmaf(x[k][v].w, w, acc[v].w);
-            }
-        }
+        for (int k = 0; k < 4; ++k) add_row(x[k], sh.w[s + k * SG]);
     }
     for (; s < nsp; s += SG) {
-        const float w = sh.w[s];
+        float4 x[VPT];
 #pragma unroll
-        for (int v = 0; v < VPT; ++v) {
-            const float4 x = load_partial4<DEVICE_COHERENT>(po + (size_t)s * (D / 4) + v * TPG + t);
-            acc[v].x = fmaf(x.x, w, acc[v].x);
-            acc[v].y = fmaf(x.y, w, acc[v].y);
-            acc[v].z = fmaf(x.z, w, acc[v].z);
-            acc[v].w = fmaf(x.w, w, acc[v].w);
-        }
+        for (int v = 0; v < VPT; ++v) x[v] = load_partial4<DEVICE_COHERENT>(po + (size_t)s * (D / 4) + v * TPG + t);
+        add_row(x, sh.w[s]);
     }
 #pragma unroll
     for (int v = 0; v < VPT; ++v) sh.acc[sg][v * TPG + t] = acc[v];

@@ -1,0 +1,133 @@
+// Measurement-only kernels (libfl_calib.so): what this machine's memory system and matrix cores sustain,
+// so that the fractions quoted for the attention kernels can be put beside a measured ceiling instead of
+// the nominal peak alone.  Nothing here is part of the attention path; libfl_decode_attn.so does not link it.
+//   fl_calib_stream_read   128-bit coalesced streaming read of a buffer, plain or non-temporal loads,
+//                          one workgroup per contiguous slice (the access pattern of the decode step)
+//   fl_calib_empty         a kernel that does nothing (launch cadence of back-to-back dependent launches)
+//   fl_calib_mfma_f16/f32  register-only loops of v_mfma_f32_32x32x16_f16 / v_mfma_f32_32x32x2_f32
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+
+template <int AUX>
+__global__ __launch_bounds__(256) void stream_read_kernel(const char *src, uint32_t bytes_per_block, float *sink)
+{
+    const char *base = src + (size_t)blockIdx.x * bytes_per_block;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(base), 0, (int)bytes_per_block, 0x00020000);
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    // eight 16-byte loads per lane in flight, 4 KB per instruction and workgroup: the streaming kernel's pattern
+    for (uint32_t off = threadIdx.x * 16u; off < bytes_per_block; off += 8u * 4096u) {
+        u32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, (uint32_t)u * 4096u, AUX);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc ^= v[u];
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[0] = 1.f; // keeps the loads alive
+}
+
+__global__ void empty_kernel() {}
+
+__device__ __forceinline__ float lane_value(uint32_t seed, bool random)
+{
+    if (!random) return 0.f;
+    uint32_t x = seed * 0x9e3779b9u + 0x7f4a7c15u;
+    x ^= x >> 16; x *= 0x85ebca6bu; x ^= x >> 13; x *= 0xc2b2ae35u; x ^= x >> 16;
+    return (float)(x & 0xffffu) * (4.0f / 65535.0f) - 2.0f; // uniform in [-2, 2]
+}
+
+__global__ __launch_bounds__(256) void mfma_f16_kernel(float *sink, int iters, int random)
+{
+    half8 a[2], b[2];
+    const uint32_t id = blockIdx.x * 256u + threadIdx.x;
+#pragma unroll
+    for (int k = 0; k < 2; ++k)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            a[k][i] = (_Float16)lane_value(id * 32u + k * 8u + i, random != 0);
+            b[k][i] = (_Float16)lane_value(id * 32u + 16u + k * 8u + i, random != 0);
+        }
+    floatx16 c[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) c[j][v] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j & 1], b[(j >> 1) & 1], c[j], 0, 0, 0);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s += c[j][v];
+    if (s == 123.456f) sink[0] = s;
+}
+
+__global__ __launch_bounds__(256) void mfma_f32_kernel(float *sink, int iters, int random)
+{
+    const uint32_t id = blockIdx.x * 256u + threadIdx.x;
+    float a[2], b[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        a[k] = lane_value(id * 4u + k, random != 0);
+        b[k] = lane_value(id * 4u + 2u + k, random != 0);
+    }
+    floatx16 c[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) c[j][v] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j & 1], b[(j >> 1) & 1], c[j], 0, 0, 0);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s += c[j][v];
+    if (s == 123.456f) sink[0] = s;
+}
+
+} // namespace
+
+extern "C" {
+
+// Reads `bytes` from src once with `blocks` workgroups of 256 threads, each over one contiguous slice;
+// bytes must be a multiple of blocks * 32768.  nontemporal: 0 plain loads, 1 `nt` loads.  Returns a hipError_t.
+int fl_calib_stream_read(const void *src, size_t bytes, int blocks, int nontemporal, float *sink, void *stream)
+{
+    if (!src || !sink || blocks <= 0 || bytes % ((size_t)blocks * 32768u) != 0 || bytes / blocks > 0x7fffffffu) return (int)hipErrorInvalidValue;
+    const uint32_t per_block = (uint32_t)(bytes / blocks);
+    if (nontemporal)
+        hipLaunchKernelGGL(stream_read_kernel<2>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const char *>(src), per_block, sink);
+    else
+        hipLaunchKernelGGL(stream_read_kernel<0>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const char *>(src), per_block, sink);
+    return (int)hipGetLastError();
+}
+
+int fl_calib_empty(void *stream)
+{
+    hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream));
+    return (int)hipGetLastError();
+}
+
+// blocks workgroups of 4 waves; every wave issues 4 * iters MFMAs.  FLOPs per launch:
+//   f16: blocks * 4 * 4 * iters * 2*32*32*16      f32: blocks * 4 * 4 * iters * 2*32*32*2
+int fl_calib_mfma(int fp32, int blocks, int iters, int random_operands, float *sink, void *stream)
+{
+    if (!sink || blocks <= 0 || iters <= 0) return (int)hipErrorInvalidValue;
+    if (fp32)
+        hipLaunchKernelGGL(mfma_f32_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), sink, iters, random_operands);
+    else
+        hipLaunchKernelGGL(mfma_f16_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), sink, iters, random_operands);
+    return (int)hipGetLastError();
+}
+
+} // extern "C"

@@ -145,6 +145,15 @@ int split_cap(const fl_attn_desc *d)
     return ragged_splits(d, d->total_len);
 }
 
+// The merge inside the streaming launch pays for small launches, where a second launch is a large part
+// of the step (B=1, H=32, ctx 4096: 15.0 us against 15.7); with thousands of workgroups the arrival round
+// trip in each of them costs more than the merge launch it saves (B=32, H=40 ragged: 214-219 us against 210).
+bool fused_merge_pays(const fl_attn_desc *d, int nsplit)
+{
+    return kWaves * 64 == flattn::kCombineThreads &&
+           (int64_t)nsplit * d->batch_size * d->head_num <= 4 * (int64_t)device_cus();
+}
+
 void make_plan(const fl_attn_desc *d, int ctx, bool ragged, fl_attn_plan *plan)
 {
     const int tile = rows_per_tile(d, unroll_for(d));
@@ -156,7 +165,7 @@ void make_plan(const fl_attn_desc *d, int ctx, bool ragged, fl_attn_plan *plan)
     plan->chunk_rows = chunk;
     plan->nsplit = (ctx + chunk - 1) / chunk;
     plan->threads = kWaves * 64;
-    plan->two_pass = plan->nsplit > 1;
+    plan->two_pass = plan->nsplit <= 1 ? 0 : (fused_merge_pays(d, plan->nsplit) ? 2 : 1);
 }
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
@@ -417,8 +426,6 @@ int fl_decode_attn_plan(const fl_attn_desc *desc, int32_t ctx, int32_t ragged, f
 
 namespace {
 
-constexpr bool kFusedMergeBuilt = kWaves * 64 == flattn::kCombineThreads;
-
 // The decode step behind every entry point.  own_scratch: take the split partials and arrival
 // counters from the library's per-GPU scratch array instead of io->workspace (no allocation either way).
 int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream, int passes, bool own_scratch)
@@ -478,8 +485,7 @@ int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_str
     }
     // One launch with the merge inside needs arrival counters that are zero: the library's own scratch
     // always is (between launches), the caller's workspace when it says so.
-    const bool fused = kFusedMergeBuilt && !direct && passes == 3 &&
-                       (own_scratch || (io->flags & FL_ATTN_IO_WORKSPACE_READY) != 0);
+    const bool fused = plan.two_pass == 2 && passes == 3 && (own_scratch || (io->flags & FL_ATTN_IO_WORKSPACE_READY) != 0);
 
     const int D = desc->size_per_head;
     Params p{};

@@ -71,9 +71,9 @@ enum { FL_ATTN_F32 = 0, FL_ATTN_F16 = 1 };
 
 /* fl_attn_io.flags.
  * FL_ATTN_IO_WORKSPACE_READY: the workspace was prepared by fl_decode_attn_workspace_init() and nothing
- * but this library has written to it since.  A step whose context is split then runs as ONE launch: the
- * workgroup that finishes the last partial of a (batch, head) pair merges them (otherwise a second,
- * small launch does). */
+ * but this library has written to it since.  A small step whose context is split (fl_attn_plan.two_pass
+ * == 2) then runs as ONE launch: the workgroup that finishes the last partial of a (batch, head) pair
+ * merges them (otherwise a second, small launch does). */
 #define FL_ATTN_IO_WORKSPACE_READY 1
 
 /* Bytes of device scratch fl_decode_attn_forward_noalloc holds per GPU. */
@@ -130,7 +130,10 @@ typedef struct fl_attn_plan {
     int32_t nsplit;       /* context splits per (b,h) */
     int32_t chunk_rows;   /* cache rows per split */
     int32_t threads;      /* threads per workgroup of the streaming kernel */
-    int32_t two_pass;     /* 1 when a combine pass follows the streaming pass */
+    int32_t two_pass;     /* 0: the context is not split.  1: split, a combine launch follows the streaming
+                             launch.  2: split and small enough that the merge runs inside the streaming
+                             launch when the workspace is ready (FL_ATTN_IO_WORKSPACE_READY) or the
+                             library's own scratch is used; a combine launch otherwise */
 } fl_attn_plan;
 
 /* Bytes of scratch fl_decode_attn_forward needs for this shape (split partials; covers every
@@ -166,7 +169,7 @@ int fl_decode_attn_workspace_init(const fl_attn_desc *desc, void *workspace, siz
  * reference, whose forward() works in the buffer carved at initialize().  Same operands, results and status
  * codes as fl_decode_attn_forward, plus FL_ATTN_ERR_SCRATCH_LIMIT when the plan of the step needs more than
  * the array holds (B * H * splits * (D + 2) * 4 bytes and B * H counters; nothing when the context is not
- * split and a float output is given).  Split steps run as one launch.  Every call on a GPU shares that
+ * split and a float output is given).  Every call on a GPU shares that
  * GPU's array: calls that may run at the same time on one GPU (two streams, two threads) race; calls in
  * stream order do not.  The first call on each GPU also looks up the array's device address
  * (hipGetSymbolAddress): make that call outside stream capture. */

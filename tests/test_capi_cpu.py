@@ -138,7 +138,7 @@ def test_plans_cover_the_context_and_respect_forced_splits():
                 assert lib.fl_decode_attn_plan(C.byref(d), ctx, ragged, C.byref(plan)) == 0
                 assert plan.nsplit >= 1 and plan.chunk_rows >= 1
                 assert plan.nsplit * plan.chunk_rows >= ctx > (plan.nsplit - 1) * plan.chunk_rows
-                assert plan.two_pass == (1 if plan.nsplit > 1 else 0)
+                assert (plan.two_pass != 0) == (plan.nsplit > 1) and plan.two_pass in (0, 1, 2)
                 cap = max(cap or 0, plan.nsplit)
         # the workspace sized from the shape alone covers the largest plan
         n = C.c_size_t(0)
@@ -159,6 +159,11 @@ def test_plan_heuristics_at_the_benchmark_shapes():
     # headline: B*H = 2048 -> single pass, no partials
     d = desc(B=64, H=32, D=128, L=2048)
     assert lib.fl_decode_attn_plan(C.byref(d), 2048, 0, C.byref(plan)) == 0 and (plan.nsplit, plan.two_pass) == (1, 0)
+    # small split launches merge inside the streaming launch (2), large ones by a second launch (1)
+    d = desc(B=1, H=32, D=128, L=4096)
+    assert lib.fl_decode_attn_plan(C.byref(d), 4096, 0, C.byref(plan)) == 0 and plan.two_pass == 2
+    d = desc(B=32, H=40, D=128, L=4096)
+    assert lib.fl_decode_attn_plan(C.byref(d), 4096, 1, C.byref(plan)) == 0 and plan.two_pass == 1
     # B=8: 256 (b,h) pairs already fill the device -> no split either
     d = desc(B=8, H=32, D=128, L=1024)
     assert lib.fl_decode_attn_plan(C.byref(d), 1024, 0, C.byref(plan)) == 0 and (plan.nsplit, plan.chunk_rows) == (1, 1024)
