@@ -302,7 +302,8 @@ hipError_t dispatch_split(int D, const Params &p, dim3 grid, hipStream_t stream)
 
 // ---- prompt phase helpers
 
-bool prefill_head_dim_ok(int D) { return D == 32 || D == 64 || D == 128; }
+bool prefill_head_dim_ok(int D) { return head_dim_ok(D); }
+constexpr bool prefill_wide(int D) { return D > 128; } // head dimension split across the waves of a workgroup
 
 // Workspace layout of the prompt phase: [float output B*H*S*D (used when the caller asks for INT8
 // only)] [mask tile classes: one word per 128-query block and 32-key tile, sized for a context that
@@ -334,20 +335,27 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
                           stream, p);
     if (e != hipSuccess) return e;
     const unsigned qblocks = (unsigned)((p.S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock);
-    const dim3 grid(qblocks * (unsigned)(p.B * p.H)); // mapped to (query block, head) by prefill_block_to_tile
     if (p.attn_mask) {
         const int ktiles = (p.start_pos + p.S + flattn::kPrefillKeysPerStep - 1) / flattn::kPrefillKeysPerStep;
         e = launch(flattn::prefill_mask_classify_kernel, dim3((unsigned)ktiles, qblocks), dim3(256), stream, p, ktiles);
         if (e != hipSuccess) return e;
     }
-    if constexpr (std::is_same<T, _Float16>::value) {
-        if (p.attn_mask && p.fast_qk) return launch(flattn::prefill_attn_f16_kernel<D, true, false>, grid, dim3(256), stream, p);
-        if (p.attn_mask) return launch(flattn::prefill_attn_f16_kernel<D, true, true>, grid, dim3(256), stream, p);
-        if (p.fast_qk) return launch(flattn::prefill_attn_f16_kernel<D, false, false>, grid, dim3(256), stream, p);
-        return launch(flattn::prefill_attn_f16_kernel<D, false, true>, grid, dim3(256), stream, p);
+    if constexpr (prefill_wide(D)) {
+        const unsigned qb32 = (unsigned)((p.S + flattn::kWideQueriesPerBlock - 1) / flattn::kWideQueriesPerBlock);
+        const dim3 wgrid(qb32 * (unsigned)(p.B * p.H)), wblock(flattn::kWideWaves * 64);
+        if (p.attn_mask) return launch(flattn::prefill_attn_wide_kernel<T, D, true>, wgrid, wblock, stream, p);
+        return launch(flattn::prefill_attn_wide_kernel<T, D, false>, wgrid, wblock, stream, p);
     } else {
-        if (p.attn_mask) return launch(flattn::prefill_attn_kernel<T, D, true>, grid, dim3(256), stream, p);
-        return launch(flattn::prefill_attn_kernel<T, D, false>, grid, dim3(256), stream, p);
+        const dim3 grid(qblocks * (unsigned)(p.B * p.H)); // mapped to (query block, head) by prefill_block_to_tile
+        if constexpr (std::is_same<T, _Float16>::value) {
+            if (p.attn_mask && p.fast_qk) return launch(flattn::prefill_attn_f16_kernel<D, true, false>, grid, dim3(256), stream, p);
+            if (p.attn_mask) return launch(flattn::prefill_attn_f16_kernel<D, true, true>, grid, dim3(256), stream, p);
+            if (p.fast_qk) return launch(flattn::prefill_attn_f16_kernel<D, false, false>, grid, dim3(256), stream, p);
+            return launch(flattn::prefill_attn_f16_kernel<D, false, true>, grid, dim3(256), stream, p);
+        } else {
+            if (p.attn_mask) return launch(flattn::prefill_attn_kernel<T, D, true>, grid, dim3(256), stream, p);
+            return launch(flattn::prefill_attn_kernel<T, D, false>, grid, dim3(256), stream, p);
+        }
     }
 }
 
@@ -358,6 +366,9 @@ hipError_t dispatch_prefill(int D, const flattn::PrefillParams &p, hipStream_t s
     case 32: return launch_prefill<T, 32>(p, stream);
     case 64: return launch_prefill<T, 64>(p, stream);
     case 128: return launch_prefill<T, 128>(p, stream);
+    case 256: return launch_prefill<T, 256>(p, stream);
+    case 512: return launch_prefill<T, 512>(p, stream);
+    case 1024: return launch_prefill<T, 1024>(p, stream);
     default: return hipErrorInvalidValue;
     }
 }
@@ -378,7 +389,7 @@ const char *fl_attn_strerror(int status)
     case FL_ATTN_OK: return "ok";
     case FL_ATTN_ERR_NULL_POINTER: return "a required pointer is NULL";
     case FL_ATTN_ERR_HEAD_DIM:
-        return "invalid size_per_head (decode step: 32, 64, 128, 256, 512, 1024; prompt phase: 32, 64, 128)";
+        return "invalid size_per_head (32, 64, 128, 256, 512 or 1024)";
     case FL_ATTN_ERR_SHAPE: return "invalid batch_size / head_num / total_len";
     case FL_ATTN_ERR_POSITION: return "start_pos or rope_row out of range for total_len";
     case FL_ATTN_ERR_WORKSPACE: return "workspace missing, too small or not 256-byte aligned";
@@ -598,7 +609,7 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     if (io->rope_row < FL_ATTN_ROPE_AT_POSITION) return FL_ATTN_ERR_POSITION;
     if (io->attn_mask && (io->mask_ld < 0 || (io->mask_ld != 0 && io->mask_ld < (int64_t)io->start_pos + seq_len)))
         return FL_ATTN_ERR_ARGUMENT;
-    if ((int64_t)desc->batch_size * desc->head_num * ((seq_len + 127) / 128) > (int64_t)INT32_MAX) return FL_ATTN_ERR_SHAPE;
+    if ((int64_t)desc->batch_size * desc->head_num * ((seq_len + 31) / 32) > (int64_t)INT32_MAX) return FL_ATTN_ERR_SHAPE;
 
     const PrefillWorkspace wl = prefill_workspace(desc, seq_len);
     if (!io->workspace || io->workspace_bytes < wl.total) return FL_ATTN_ERR_WORKSPACE;

@@ -168,7 +168,7 @@ namespace FasterLLaMA
         /**
          * key_cache_, value_cache_: [batch_size, head_num, total_len_, size_per_head]
          * freq_cis: [rows >= start_pos + seq_len, size_per_head]
-         * seq_len == 1: decode step; 1 < seq_len <= max_prompt_len: prompt phase (size_per_head 32/64/128).
+         * seq_len == 1: decode step; 1 < seq_len <= max_prompt_len: prompt phase.
          */
         void forward(const DataType_ *from_tensor, const float *freq_cis, float *key_cache_, float *value_cache_,
                      DataType_ *decoder_output, const int start_pos, const int seq_len);

@@ -764,6 +764,175 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     }
 }
 
+// ---------------------------------------------------------------- head sizes 256 / 512 / 1024
+
+// The reference serves size_per_head 256, 512 and 1024 as well (decoder_kernels.cu:474-551, :588).  With
+// such rows the per-wave state of the kernels above (rotated queries and output accumulators of 32 queries)
+// no longer fits the register file, so here the HEAD DIMENSION is split across the waves of a workgroup:
+// a workgroup of 8 waves owns 32 queries of one (b,h); wave w owns the DW = D/8 dims [w*DW, (w+1)*DW).
+//   scores   every wave forms the partial S^T = K[:, its dims] Q^T[its dims, :] of the 32-key tile; the
+//            eight partials meet in LDS and every wave adds them up in the same order, so all waves hold
+//            the same scores and run the same softmax (decoder_kernels.cu:811-833, expf, true division);
+//   output   O^T[its dims, :] += V^T[its dims, :] P^T, in registers until the end.
+// FP32 MFMA (v_mfma_f32_32x32x2_f32) for both cache types — fp16 rows are widened on load, their products
+// are exact — which keeps the 1e-5 bar of the FP32 path and needs no transposing reads: K and V operands
+// come straight from global memory (K: 16 bytes of one row per lane, V: 32 consecutive elements of one
+// row per half-wave), nothing is staged.  Mask tile classes as above.  Slower than the kernels for the
+// common head sizes by design: correctness first for shapes no LLaMA model uses.
+constexpr int kWideWaves = 8;
+constexpr int kWideQueriesPerBlock = 32;
+
+template <typename T, int D, bool HAS_MASK>
+__global__ __launch_bounds__(kWideWaves * 64) void prefill_attn_wide_kernel(const PrefillParams p)
+{
+    constexpr int BN = kPrefillKeysPerStep;
+    constexpr int DW = D / kWideWaves; // dims per wave: 32, 64 or 128
+    constexpr int NC = DW / 8, NDT = DW / 32;
+    static_assert(DW % 32 == 0, "each wave owns whole 32-column output tiles");
+
+    __shared__ float s_part[2][kWideWaves][16][64]; // partial score tiles of two consecutive key tiles
+
+    const int S = p.S, P = p.start_pos, L = p.L;
+    const int ctx = P + S;
+    const int QB = (S + kWideQueriesPerBlock - 1) / kWideQueriesPerBlock;
+    const int BH = p.B * p.H;
+    const int bh = (int)blockIdx.x % BH;
+    const int qb = QB - 1 - (int)blockIdx.x / BH; // long query blocks first under a causal mask
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int qi = lane & 31, hf = lane >> 5;
+    const int q_row = qb * kWideQueriesPerBlock + qi;
+    const bool q_ok = q_row < S;
+    const int d_wave = wave * DW;
+
+    float qreg[NC][4];
+    {
+        const int64_t token = (int64_t)(bh / p.H) * S + (q_ok ? q_row : 0);
+        const int row = (p.rope_row < 0 ? P : p.rope_row) + (q_ok ? q_row : 0);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            rotated_query_chunk<T, 4>(p, D, token, bh % p.H, d_wave + 8 * c + 4 * hf, row, qreg[c]);
+            if (!q_ok) qreg[c][0] = qreg[c][1] = qreg[c][2] = qreg[c][3] = 0.f;
+        }
+    }
+
+    floatx16 ot[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) ot[dt][v] = 0.f;
+    float m = kMaxFloor, l = 0.f;
+    const float *mrow = HAS_MASK ? p.attn_mask + (size_t)(P + (q_ok ? q_row : 0)) * p.mask_ld : nullptr;
+    const T *Kb = reinterpret_cast<const T *>(p.k_cache) + (size_t)bh * L * D;
+    const T *Vb = reinterpret_cast<const T *>(p.v_cache) + (size_t)bh * L * D;
+    const float scale = p.scale;
+    const int NT = (ctx + BN - 1) / BN;
+    // class of this 32-query block per key tile: byte (qb % 4) of the word of its 128-query block
+    const uint32_t *cls = HAS_MASK ? p.tile_class + (size_t)(qb / 4) * NT : nullptr;
+
+    int buf = 0;
+    for (int t = 0; t < NT; ++t) {
+        uint32_t tc = kTileZero;
+        if constexpr (HAS_MASK) {
+            tc = (__builtin_amdgcn_readfirstlane(cls[t]) >> (8 * (qb & 3))) & 0xffu;
+            if (tc == kTileSkip) continue; // uniform over the workgroup: every wave skips the same tiles
+        }
+        const int k0 = t * BN;
+
+        // partial S^T over this wave's dims: keys k0 + qi (rows), queries (columns)
+        floatx16 st;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) st[v] = 0.f;
+        {
+            const int key = k0 + qi;
+            const T *krow = Kb + (size_t)(key < ctx ? key : 0) * D + d_wave + 4 * hf;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                float ka[4];
+                if constexpr (std::is_same<T, float>::value) {
+                    const float4 x = *reinterpret_cast<const float4 *>(krow + 8 * c);
+                    ka[0] = x.x; ka[1] = x.y; ka[2] = x.z; ka[3] = x.w;
+                } else {
+                    const half4 x = *reinterpret_cast<const half4 *>(krow + 8 * c);
+                    ka[0] = (float)x[0]; ka[1] = (float)x[1]; ka[2] = (float)x[2]; ka[3] = (float)x[3];
+                }
+                if (key >= ctx) ka[0] = ka[1] = ka[2] = ka[3] = 0.f; // rows past the context may hold anything
+#pragma unroll
+                for (int r = 0; r < 4; ++r) st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[r], qreg[c][r], st, 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s_part[buf][wave][v][lane] = st[v];
+        __syncthreads(); // the buffer written two tiles ago was read before the previous tile's barrier
+        float sc[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            float x = s_part[buf][0][v][lane];
+#pragma unroll
+            for (int w = 1; w < kWideWaves; ++w) x += s_part[buf][w][v][lane];
+            sc[v] = x;
+        }
+        // v = qk * scale + mask (decoder_kernels.cu:815); fma(s, scale, 0) == s * scale, so tiles whose mask
+        // entries are all zero take the short way
+        if (HAS_MASK && tc == kTileMixed) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) sc[v] = fmaf(sc[v], scale, mrow[min(k0 + 8 * (v / 4) + 4 * hf + (v % 4), ctx - 1)]);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) sc[v] *= scale;
+        }
+        float mx = m;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            if (k0 + 8 * (v / 4) + 4 * hf + (v % 4) >= ctx) sc[v] = -__builtin_inff();
+            mx = fmaxf(mx, sc[v]);
+        }
+        buf ^= 1;
+        mx = fmaxf(mx, __shfl_xor(mx, 32)); // the other half-wave holds the other 16 keys of this query
+        const float alpha = expf(m - mx);
+        m = mx;
+        l *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) ot[dt][v] *= alpha;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            sc[v] = expf(sc[v] - m);
+            l += sc[v];
+        }
+
+        // O^T[this wave's dims] += V^T P^T: two keys per MFMA; step s of half hf is key 8*(s/4) + 4*hf + s%4,
+        // the key whose probability this lane holds in sc[s]
+#pragma unroll
+        for (int s4 = 0; s4 < 16; ++s4) {
+            const int key = k0 + 8 * (s4 / 4) + 4 * hf + (s4 % 4);
+            const T *vrow = Vb + (size_t)(key < ctx ? key : 0) * D + d_wave + qi;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                float va = (float)vrow[32 * dt];
+                if (key >= ctx) va = 0.f;
+                ot[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(va, sc[s4], ot[dt], 0, 0, 0);
+            }
+        }
+    }
+
+    l += __shfl_xor(l, 32);
+    if (q_ok) {
+        float *dst = p.out + ((size_t)bh * S + q_row) * D + d_wave;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                float4 r;
+                r.x = ot[dt][4 * g4 + 0] / l; // p = e / sum (decoder_kernels.cu:833)
+                r.y = ot[dt][4 * g4 + 1] / l;
+                r.z = ot[dt][4 * g4 + 2] / l;
+                r.w = ot[dt][4 * g4 + 3] / l;
+                *reinterpret_cast<float4 *>(dst + 32 * dt + 8 * g4 + 4 * hf) = r;
+            }
+    }
+}
+
 // ---------------------------------------------------------------- INT8 epilogue with transpose
 
 // grid = B*S, block = 1024.  attn [B,H,S,D] float -> out_q [B,S,H*D] int8, out_scale [B,S]

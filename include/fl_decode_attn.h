@@ -188,7 +188,9 @@ int fl_decode_attn_forward_noalloc(const fl_attn_desc *desc, const fl_attn_io *i
  * start_pos_per_seq must be NULL.  Keys are the cache rows [0, start_pos + seq_len) after the append.
  * 32 x 32 tiles of the mask whose entries are all <= -1e30 (the -FLT_MAX of samples/llama_fp16.cu:73-81)
  * are not multiplied: with finite K and V their weights are exactly 0, so no bit of the output changes.
- * size_per_head must be 32, 64 or 128.  Workspace: fl_prefill_attn_workspace_bytes(). */
+ * Every size_per_head of the decode step is served; 256, 512 and 1024 by a kernel that splits the head
+ * dimension across the waves of a workgroup (FP32 matrix instructions for both cache types).  Workspace:
+ * fl_prefill_attn_workspace_bytes(). */
 int fl_prefill_attn_workspace_bytes(const fl_attn_desc *desc, int32_t seq_len, size_t *bytes);
 int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int32_t seq_len,
                             void *hip_stream);

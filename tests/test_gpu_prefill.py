@@ -68,10 +68,54 @@ def test_prefill_matches_oracle(gpu, dtype, S, P):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
-@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("D", [32, 64, 128, 256, 512, 1024])
 def test_prefill_head_sizes_and_no_mask(gpu, dtype, D):
+    # the reference's set of head sizes (decoder_kernels.cu:474-551, :588), plus 32
     out, want, _ = run_both(gpu, 2, 5, D, 256, 77, 10, dtype, mask=None, seed=D)
     close(out, want, dtype, f"D={D} no mask")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+@pytest.mark.parametrize("D", [256, 512, 1024])
+@pytest.mark.parametrize("S,P", [(1, 0), (33, 0), (130, 61), (64, 192)])
+def test_prefill_wide_heads_with_masks(gpu, dtype, D, S, P):
+    """Head sizes above 128 (the head dimension is split across the waves of a workgroup): ragged query
+    blocks, chunked prompts, the -1e5 causal mask (every tile evaluated) and the -FLT_MAX one (tiles dropped)."""
+    L = 256
+    for fill in (-1e5, -FMAX):
+        out, want, _ = run_both(gpu, 2, 3, D, L, S, P, dtype, mask=causal_mask(L, fill), seed=D + S + P)
+        close(out, want, dtype, f"D={D} S={S} P={P} fill={fill}")
+
+
+def test_prefill_wide_heads_dense_mask_scaled_keys_and_decode_handover(gpu):
+    """D = 256: a dense random mask with an odd row stride, key rows scaled by 8, then decode steps on the
+    caches the prompt phase wrote (bit-identical rows)."""
+    import torch
+    from fasterllama_amd.decode_attn import DecodeAttention, PrefillAttention
+    B, H, D, L, S, ld = 2, 3, 256, 160, 100, 171
+    for dtype in ("f16", "f32"):
+        tdt = torch.float16 if dtype == "f16" else torch.float32
+        q, k, v, kc, vc, f = make(B, H, D, L, S, dtype, 91)
+        k[:, 17] *= 8
+        k[:, 70] *= 8
+        mask = (np.random.default_rng(2).standard_normal((L, ld)) * 3).astype(np.float32)
+        kc_ref, vc_ref = kc.copy(), vc.copy()
+        want = ref.prefill_attn(q, k, v, kc_ref, vc_ref, f, attn_mask=mask, mask_ld=ld, acc_double=True, threads=16)
+        t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+        op = PrefillAttention(B, H, D, L, S, tdt, device=gpu)
+        kc_d, vc_d = t(kc), t(vc)
+        out = op.prefill(t(q), t(k), t(v), kc_d, vc_d, t(f), attn_mask=t(mask), mask_ld=ld)
+        torch.cuda.synchronize()
+        assert_cache_bit_exact(kc_d.cpu().numpy(), kc_ref, "k_cache")
+        assert_out_close(out.cpu().numpy(), want, dtype, f"wide dense mask {dtype}",
+                         float_ref=lambda: ref.prefill_attn(q, k, v, kc.copy(), vc.copy(), f, attn_mask=mask, mask_ld=ld, threads=16))
+        dec = DecodeAttention(B, H, D, L, tdt, device=gpu)
+        for step in range(3):
+            qs, ks, vs, _, _, _ = make(B, H, D, L, 1, dtype, 200 + step)
+            w = ref.decode_attn(qs, ks, vs, kc_ref, vc_ref, f, start_pos=S + step, acc_double=True)
+            g = dec.forward(t(qs), t(ks), t(vs), kc_d, vc_d, t(f), start_pos=S + step)
+            assert_out_close(g.cpu().numpy(), w, dtype, f"decode step {step} after a wide prompt", head_dim=D)
+        assert_cache_bit_exact(kc_d.cpu().numpy(), kc_ref, "k_cache after decode steps")
 
 
 def test_prefill_strict_mask_first_row_is_nan(gpu):
@@ -332,7 +376,7 @@ def test_prefill_argument_errors(gpu):
     import torch
     from fasterllama_amd.decode_attn import PrefillAttention
     with pytest.raises(capi.FlAttnError) as e:
-        PrefillAttention(1, 2, 256, 64, 16, torch.float16, device=gpu)
+        PrefillAttention(1, 2, 96, 64, 16, torch.float16, device=gpu)
     assert e.value.status == capi.FL_ATTN_ERR_HEAD_DIM
     op = PrefillAttention(1, 2, 64, 64, 16, torch.float16, device=gpu)
     z = torch.zeros(1, 16, 2, 64, dtype=torch.float16, device=gpu)
