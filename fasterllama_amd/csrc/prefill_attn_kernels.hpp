@@ -420,6 +420,13 @@ template <int D, bool HAS_MASK, bool QSPLIT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8)))
 void prefill_attn_f16_kernel(const PrefillParams p)
 {
+    // Operand prefetch.  Where the kernel runs two waves per SIMD anyway, all K operands of a tile are read
+    // from LDS before the first product is issued (and, with the single fp16 query, the V operands before the
+    // softmax), so LDS latency is paid once per tile and not once per pair of matrix instructions.  The
+    // unmasked single-query instance is left alone: it fits 168 registers, runs THREE waves per SIMD and
+    // loses more from a fourth dozen of registers than it gains (B=8, S=1024: 0.221 ms against 0.240).
+    constexpr bool PF_KA = HAS_MASK || QSPLIT;
+    constexpr bool PF_VA = HAS_MASK && !QSPLIT;
     constexpr int BN = kPrefillKeysPerStep; // 32
     constexpr int LDK = D + 8;              // halfs; rows start 4 banks apart (128-bit operand reads)
     constexpr int LDV = D + 32;             // halfs; rows start 16 banks apart (8 rows x 64 bytes per transposing read)
@@ -543,38 +550,38 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     const _Float16 *Kb = reinterpret_cast<const _Float16 *>(p.k_cache) + (size_t)bh * L * D;
     const _Float16 *Vb = reinterpret_cast<const _Float16 *>(p.v_cache) + (size_t)bh * L * D;
 
-    // global -> registers (fetch) and registers -> LDS (commit) of one key tile
+    // global -> registers (fetch) and registers -> LDS (commit) of one key tile.  Raw buffer loads whose
+    // descriptors end at the context's last row: a row at or beyond the context — it may hold anything —
+    // arrives as zeros by the hardware's range check, with no branch, and the addresses are one scalar
+    // base plus one 32-bit offset per chunk.
     half8 kstage[LPT], vstage[LPT];
     constexpr bool EXACT = (BN * CPR) % 256 == 0; // every thread owns LPT chunks of each matrix
+    const __amdgpu_buffer_rsrc_t Kbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16 *>(Kb), 0, (int)((uint32_t)ctx * (uint32_t)(D * 2)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t Vbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16 *>(Vb), 0, (int)((uint32_t)ctx * (uint32_t)(D * 2)), 0x00020000);
+    uint32_t src_off[LPT], k_dst[LPT], v_dst[LPT]; // byte offsets: in a 32-row slab of the cache, in the LDS tiles
+#pragma unroll
+    for (int j = 0; j < LPT; ++j) {
+        const int idx = tid + j * 256;
+        const int r = idx / CPR, cc = idx % CPR;
+        src_off[j] = (EXACT || idx < BN * CPR) ? (uint32_t)(r * D * 2 + cc * 16) : kLaneOutOfRange;
+        k_dst[j] = (uint32_t)((r * LDK + cc * 8) * 2);
+        v_dst[j] = (uint32_t)((2 * BN * LDK + r * LDV + cc * 8) * 2);
+    }
     auto fetch = [&](int t) {
-        const int k0 = t * BN;
-        const bool tail = k0 + BN > ctx;
+        const uint32_t slab = (uint32_t)t * (uint32_t)(BN * D * 2); // uniform; part of the checked offset
 #pragma unroll
         for (int j = 0; j < LPT; ++j) {
-            const int idx = tid + j * 256;
-            const int r = idx / CPR, cc = idx % CPR;
-            if (!tail) {
-                if (EXACT || idx < BN * CPR) {
-                    kstage[j] = *reinterpret_cast<const half8 *>(Kb + (size_t)(k0 + r) * D + cc * 8);
-                    vstage[j] = *reinterpret_cast<const half8 *>(Vb + (size_t)(k0 + r) * D + cc * 8);
-                }
-            } else { // rows beyond the context may hold anything: they enter as zeros
-#pragma unroll
-                for (int i = 0; i < 8; ++i) kstage[j][i] = vstage[j][i] = (_Float16)0;
-                if ((EXACT || idx < BN * CPR) && k0 + r < ctx) {
-                    kstage[j] = *reinterpret_cast<const half8 *>(Kb + (size_t)(k0 + r) * D + cc * 8);
-                    vstage[j] = *reinterpret_cast<const half8 *>(Vb + (size_t)(k0 + r) * D + cc * 8);
-                }
-            }
+            kstage[j] = __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(Kbuf, src_off[j] + slab, 0, 0));
+            vstage[j] = __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(Vbuf, src_off[j] + slab, 0, 0));
         }
     };
     auto commit = [&](int buf) {
+        char *base = reinterpret_cast<char *>(smem);
 #pragma unroll
         for (int j = 0; j < LPT; ++j) {
-            const int idx = tid + j * 256;
-            if (EXACT || idx < BN * CPR) {
-                *reinterpret_cast<half8 *>(&sK[buf][idx / CPR][(idx % CPR) * 8]) = kstage[j];
-                *reinterpret_cast<half8 *>(&sV[buf][idx / CPR][(idx % CPR) * 8]) = vstage[j];
+            if (EXACT || tid + j * 256 < BN * CPR) {
+                *reinterpret_cast<half8 *>(base + k_dst[j] + (uint32_t)(buf * BN * LDK * 2)) = kstage[j];
+                *reinterpret_cast<half8 *>(base + v_dst[j] + (uint32_t)(buf * BN * LDV * 2)) = vstage[j];
             }
         }
     };
@@ -605,8 +612,10 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         fetch((int)(e0 >> 8));
         commit(0);
         if (n > 1) fetch((int)(e1 >> 8));
-        int buf = 0;
-        for (int i = 0; i < n; ++i) {
+        // one tile of the pipeline; the LDS buffer index is a compile-time constant (the loop below is
+        // unrolled by two), so every LDS address is a register plus an immediate
+        auto tile_step = [&](int i, auto buf_tag) {
+            constexpr int buf = decltype(buf_tag)::value;
             const int t = (int)(e0 >> 8);
             __syncthreads(); // tile t is visible; every wave is done with the other buffer
 
@@ -649,7 +658,15 @@ void prefill_attn_f16_kernel(const PrefillParams p)
             }
 
             if (tc != kTileSkip) {
-                const half8 ka0 = *reinterpret_cast<const half8 *>(&sK[buf][qi][8 * hf]);
+                half8 kall[PF_KA ? NC : 1];
+                if constexpr (PF_KA) {
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) kall[c] = *reinterpret_cast<const half8 *>(&sK[buf][qi][16 * c + 8 * hf]);
+                    __builtin_amdgcn_sched_barrier(0);
+                } else {
+                    kall[0] = *reinterpret_cast<const half8 *>(&sK[buf][qi][8 * hf]);
+                }
+                const half8 ka0 = kall[0];
                 if (special) {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
@@ -669,11 +686,22 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 if constexpr (QSPLIT) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka0, qlo[0], st, 0, 0, 0);
 #pragma unroll
                 for (int c = 1; c < NC; ++c) {
-                    const half8 ka = *reinterpret_cast<const half8 *>(&sK[buf][qi][16 * c + 8 * hf]);
+                    const half8 ka = PF_KA ? kall[PF_KA ? c : 0] : *reinterpret_cast<const half8 *>(&sK[buf][qi][16 * c + 8 * hf]);
                     st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[c], st, 0, 0, 0);
                     if constexpr (QSPLIT) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qlo[c], st, 0, 0, 0);
                 }
 
+                half4 vlo[PF_VA ? NDT : 1][2], vhi[PF_VA ? NDT : 1][2];
+                if constexpr (PF_VA) {
+#pragma unroll
+                    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                        for (int u = 0; u < 2; ++u) {
+                            vlo[dt][u] = lds_read_tr16(&sV[buf][16 * u + vrow][32 * dt + vcol]);
+                            vhi[dt][u] = lds_read_tr16(&sV[buf][16 * u + 8 + vrow][32 * dt + vcol]);
+                        }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 // Softmax update of this lane's query (decoder_kernels.cu:811-833 in base 2).  The reference
                 // maximum m may lag the true running maximum by up to kLazyMax (weights up to 2^kLazyMax,
                 // well inside fp16 and exact in the final ratio): with 32 queries per wave some maximum
@@ -707,8 +735,8 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                     for (int u = 0; u < 2; ++u) {
-                        const half4 lo = lds_read_tr16(&sV[buf][16 * u + vrow][32 * dt + vcol]);
-                        const half4 hi = lds_read_tr16(&sV[buf][16 * u + 8 + vrow][32 * dt + vcol]);
+                        const half4 lo = PF_VA ? vlo[PF_VA ? dt : 0][u] : lds_read_tr16(&sV[buf][16 * u + vrow][32 * dt + vcol]);
+                        const half4 hi = PF_VA ? vhi[PF_VA ? dt : 0][u] : lds_read_tr16(&sV[buf][16 * u + 8 + vrow][32 * dt + vcol]);
                         half8 va;
                         va[0] = lo[0]; va[1] = lo[1]; va[2] = lo[2]; va[3] = lo[3];
                         va[4] = hi[0]; va[5] = hi[1]; va[6] = hi[2]; va[7] = hi[3];
@@ -720,7 +748,10 @@ void prefill_attn_f16_kernel(const PrefillParams p)
             e1 = e2;
             e2 = __builtin_amdgcn_readfirstlane(e3);
             e3 = i + 4 < n ? list_entry(c0, i + 4) : 0u;
-            buf ^= 1;
+        };
+        for (int i = 0; i < n; i += 2) {
+            tile_step(i, std::integral_constant<int, 0>{});
+            if (i + 1 < n) tile_step(i + 1, std::integral_constant<int, 1>{});
         }
     }
 
