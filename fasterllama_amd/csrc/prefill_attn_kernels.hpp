@@ -98,11 +98,12 @@ __global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillP
 // RoPE(q) for N consecutive head dims d0.. of one prompt token, in FP32: the attention kernels
 // rotate their own queries while they load them (decoder_kernels.cu:449-458), so the rotated
 // queries never travel through memory.  `token` indexes [B,S], `row` is the table row.
-template <typename T, int N>
+// I32: 1 / 0 when the caller has already branched on the input format (int32 accumulators or not), -1 to test here.
+template <typename T, int N, int I32 = -1>
 __device__ __forceinline__ void rotated_query_chunk(const PrefillParams &p, int D, int64_t token, int h, int d0, int row,
                                                     float (&out)[N])
 {
-    const bool is_i32 = p.inp_scale != nullptr;
+    const bool is_i32 = I32 < 0 ? p.inp_scale != nullptr : I32 != 0;
     float x[N];
     load_token_chunk<T, N>(p.q, (size_t)(token * p.H + h) * D + d0, is_i32, is_i32 ? p.inp_scale[token] : 0.f,
                            is_i32 ? p.wq_scale + h * D + d0 : nullptr, x);
@@ -489,64 +490,6 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         else return (uint32_t)(c0 + i) << 8 | 0x55u;
     };
 
-    // Rotated queries of the workgroup: loaded and rotated cooperatively (16 lanes per 256-byte row, so
-    // the [B,S,H,D] rows are read whole), rounded once to fp16 as MFMA operands, and handed to their
-    // lanes through LDS.  Reading them per lane instead — 32 rows a wave, 16 bytes a lane — keeps the
-    // texture units busy for longer than ten key tiles take.
-    half8 qreg[NC];
-    half8 qlo[QSPLIT ? NC : 1]; // remainders q - fp16(q): the first product runs on the pair, see below
-    {
-        const int b = bh / p.H, h = bh % p.H;
-        const int row0 = p.rope_row < 0 ? P : p.rope_row;
-        constexpr int QPT = kPrefillQueriesPerBlock * CPR / 256; // 16-byte chunks per thread
-        half8 lo_keep[QSPLIT ? QPT : 1];
-#pragma unroll
-        for (int j = 0; j < QPT; ++j) {
-            const int idx = tid + j * 256;
-            const int r = idx / CPR, cc = idx % CPR;
-            const int q = qb * kPrefillQueriesPerBlock + r;
-            half8 hq;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) hq[i] = (_Float16)0;
-            if constexpr (QSPLIT) lo_keep[j] = hq;
-            if (q < S) {
-                float x[8];
-                rotated_query_chunk<_Float16, 8>(p, D, (int64_t)b * S + q, h, cc * 8, row0 + q, x);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    hq[i] = (_Float16)x[i];
-                    if constexpr (QSPLIT) lo_keep[j][i] = (_Float16)(x[i] - (float)hq[i]);
-                }
-            }
-            *reinterpret_cast<half8 *>(smem + r * LDQ + cc * 8) = hq;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int c = 0; c < NC; ++c)
-            qreg[c] = *reinterpret_cast<const half8 *>(smem + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
-        __syncthreads();
-        if constexpr (QSPLIT) {
-#pragma unroll
-            for (int j = 0; j < QPT; ++j) {
-                const int idx = tid + j * 256;
-                *reinterpret_cast<half8 *>(smem + (idx / CPR) * LDQ + (idx % CPR) * 8) = lo_keep[j];
-            }
-            __syncthreads();
-#pragma unroll
-            for (int c = 0; c < NC; ++c)
-                qlo[c] = *reinterpret_cast<const half8 *>(smem + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
-            __syncthreads();
-        }
-        // the tile buffers are free for K and V
-    }
-
-    floatx16 ot[NDT];
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) ot[dt][v] = 0.f;
-    const float scale = p.scale * kLog2e;
-    float m = kMaxFloor * kLog2e, l = 0.f;
     const _Float16 *Kb = reinterpret_cast<const _Float16 *>(p.k_cache) + (size_t)bh * L * D;
     const _Float16 *Vb = reinterpret_cast<const _Float16 *>(p.v_cache) + (size_t)bh * L * D;
 
@@ -586,6 +529,79 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         }
     };
 
+    // The list of the first chunk and its first tile are requested BEFORE the queries: the class words, the
+    // first K/V tile and the queries then travel together instead of one memory round trip after the other.
+    const int first_c1 = min(kTileListCap, NT);
+    int n_first = first_c1;
+    if constexpr (HAS_MASK) n_first = build_list(0, first_c1);
+    if (n_first > 0) fetch((int)(__builtin_amdgcn_readfirstlane(list_entry(0, 0)) >> 8));
+
+    // Rotated queries of the workgroup: loaded and rotated cooperatively (16 lanes per 256-byte row, so
+    // the [B,S,H,D] rows are read whole), rounded once to fp16 as MFMA operands, and handed to their
+    // lanes through LDS.  Reading them per lane instead — 32 rows a wave, 16 bytes a lane — keeps the
+    // texture units busy for longer than ten key tiles take.
+    half8 qreg[NC];
+    half8 qlo[QSPLIT ? NC : 1]; // remainders q - fp16(q): the first product runs on the pair, see below
+    {
+        const int b = bh / p.H, h = bh % p.H;
+        const int row0 = p.rope_row < 0 ? P : p.rope_row;
+        constexpr int QPT = kPrefillQueriesPerBlock * CPR / 256; // 16-byte chunks per thread
+        half8 lo_keep[QSPLIT ? QPT : 1];
+        // Every chunk is loaded unconditionally (rows past the prompt read the prompt's last row and are
+        // zeroed afterwards): with the loads under a branch the compiler waits for each chunk before it
+        // requests the next, eight memory round trips in a row (11 us per workgroup instead of 2.5).
+        float x[QPT][8];
+        auto load_queries = [&](auto i32_tag) { // one straight run of loads per input format
+#pragma unroll
+            for (int j = 0; j < QPT; ++j) {
+                const int idx = tid + j * 256;
+                const int r = idx / CPR, cc = idx % CPR;
+                const int q = min(qb * kPrefillQueriesPerBlock + r, S - 1);
+                rotated_query_chunk<_Float16, 8, decltype(i32_tag)::value>(p, D, (int64_t)b * S + q, h, cc * 8, row0 + q, x[j]);
+            }
+        };
+        if (p.inp_scale != nullptr) load_queries(std::integral_constant<int, 1>{});
+        else load_queries(std::integral_constant<int, 0>{});
+#pragma unroll
+        for (int j = 0; j < QPT; ++j) {
+            const int idx = tid + j * 256;
+            const int r = idx / CPR, cc = idx % CPR;
+            const bool valid = qb * kPrefillQueriesPerBlock + r < S;
+            half8 hq;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                hq[i] = valid ? (_Float16)x[j][i] : (_Float16)0;
+                if constexpr (QSPLIT) lo_keep[j][i] = valid ? (_Float16)(x[j][i] - (float)hq[i]) : (_Float16)0;
+            }
+            *reinterpret_cast<half8 *>(smem + r * LDQ + cc * 8) = hq;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+            qreg[c] = *reinterpret_cast<const half8 *>(smem + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
+        __syncthreads();
+        if constexpr (QSPLIT) {
+#pragma unroll
+            for (int j = 0; j < QPT; ++j) {
+                const int idx = tid + j * 256;
+                *reinterpret_cast<half8 *>(smem + (idx / CPR) * LDQ + (idx % CPR) * 8) = lo_keep[j];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+                qlo[c] = *reinterpret_cast<const half8 *>(smem + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
+            __syncthreads();
+        }
+        // the tile buffers are free for K and V
+    }
+
+    floatx16 ot[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) ot[dt][v] = 0.f;
+    const float scale = p.scale * kLog2e;
+    float m = kMaxFloor * kLog2e, l = 0.f;
     // per-lane source of the transposing V reads: row 4hf + (lane%16)/4, halfs 16*((lane/16)%2) + 4*(lane%4)
     const int vrow = 4 * hf + ((lane & 15) >> 2), vcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
     const float inv_scale = 1.0f / p.scale;
@@ -602,14 +618,15 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     for (int c0 = 0; c0 < NT; c0 += kTileListCap) {
         const int c1 = min(c0 + kTileListCap, NT);
         int n = c1 - c0;
-        if constexpr (HAS_MASK) n = build_list(c0, c1); // ends with a barrier: the tile buffers are free again
-        else if (c0 > 0) __syncthreads();
+        if (c0 == 0) n = n_first; // built, and its first tile requested, before the queries were loaded
+        else if constexpr (HAS_MASK) n = build_list(c0, c1); // ends with a barrier: the tile buffers are free again
+        else __syncthreads();
         if (n == 0) continue;
         uint32_t e0 = __builtin_amdgcn_readfirstlane(list_entry(c0, 0));
         uint32_t e1 = n > 1 ? __builtin_amdgcn_readfirstlane(list_entry(c0, 1)) : 0u;
         uint32_t e2 = n > 2 ? __builtin_amdgcn_readfirstlane(list_entry(c0, 2)) : 0u;
         uint32_t e3 = n > 3 ? list_entry(c0, 3) : 0u;
-        fetch((int)(e0 >> 8));
+        if (c0 > 0) fetch((int)(e0 >> 8));
         commit(0);
         if (n > 1) fetch((int)(e1 >> 8));
         // one tile of the pipeline; the LDS buffer index is a compile-time constant (the loop below is
