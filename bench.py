@@ -91,7 +91,13 @@ def bench_prefill(args) -> int:
     vc = torch.zeros_like(kc)
     out = torch.empty(B, H, S, D, dtype=torch.float32, device=dev)
     op = PrefillAttention(B, H, D, L, S, t_dt, device=dev, fast_qk=args.prefill_fast_qk)
-    io = op.make_io(q, k, v, kc, vc, freq, out, start_pos=P, attn_mask=None if args.prefill_mask == "none" else mask)
+    # the reference installs ONE mask for every layer and call (samples/llama_fp16.cu:139-150): its tile classes are
+    # computed once, outside the timed step (fl_prefill_mask_classify), unless --prefill-classify-per-call
+    table = None
+    if args.prefill_mask != "none" and not args.prefill_classify_per_call:
+        table = op.classify_mask(mask)
+    io = op.make_io(q, k, v, kc, vc, freq, out, start_pos=P, attn_mask=None if args.prefill_mask == "none" else mask,
+                    mask_tile_classes=table)
     stream = torch.cuda.current_stream(dev)
 
     def run(n):
@@ -146,7 +152,8 @@ def bench_prefill(args) -> int:
                                   "causal-1e5": "causal additive mask, -1e5 above the diagonal",
                                   "block-causal": "additive mask, causal over blocks of 128 tokens, -FLT_MAX above",
                                   "none": "no mask"}[args.prefill_mask]
-                               + (", fast first product (fp16 queries)" if args.prefill_fast_qk and w["dtype"] == "f16" else ""),
+                               + (", fast first product (fp16 queries)" if args.prefill_fast_qk and w["dtype"] == "f16" else "")
+                               + (", mask tiles classified once per mask" if table is not None else ""),
                    "flops_per_step": flops, "dense_flops_per_step": dense_flops,
                    "tokens_per_s": round(B * S / (ms * 1e-3), 1)},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": peak, "unit": "TFLOP/s",
@@ -492,6 +499,8 @@ def main() -> int:
     ap.add_argument("--prefill-mask", default="causal", choices=["causal", "causal-1e5", "block-causal", "none"],
                     help="prompt-phase workloads: additive causal mask with -FLT_MAX (the reference's driver) or "
                          "-1e5 (its kernel harness) above the diagonal, or no mask")
+    ap.add_argument("--prefill-classify-per-call", action="store_true",
+                    help="prompt-phase workloads: classify the mask's tiles inside every step instead of once per mask")
     ap.add_argument("--prefill-fast-qk", action="store_true",
                     help="prompt-phase fp16 workloads: FL_ATTN_FLAG_FAST_PROMPT_QK (queries as one fp16 value)")
     ap.add_argument("--mask", default="none", choices=["none", "causal", "strict"],

@@ -40,6 +40,8 @@ EXPORTED_SYMBOLS = (
     "fl_decode_attn_workspace_init",
     "fl_prefill_attn_workspace_bytes",
     "fl_prefill_attn_forward",
+    "fl_prefill_mask_classes_bytes",
+    "fl_prefill_mask_classify",
     "fl_rope_table",
     "fl_kv_cache_bytes",
     "fl_attn_strerror",
@@ -85,6 +87,7 @@ class AttnIO(C.Structure):
         ("v_weight_scale", C.c_void_p),
         ("out_int8", C.c_void_p),
         ("out_scale", C.c_void_p),
+        ("mask_tile_classes", C.c_void_p),
     ]
 
 
@@ -134,6 +137,10 @@ def load() -> C.CDLL:
     lib.fl_prefill_attn_workspace_bytes.restype = C.c_int
     lib.fl_prefill_attn_forward.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnIO), C.c_int32, C.c_void_p]
     lib.fl_prefill_attn_forward.restype = C.c_int
+    lib.fl_prefill_mask_classes_bytes.argtypes = [C.POINTER(AttnDesc), C.POINTER(C.c_size_t)]
+    lib.fl_prefill_mask_classes_bytes.restype = C.c_int
+    lib.fl_prefill_mask_classify.argtypes = [C.POINTER(AttnDesc), C.c_void_p, C.c_int64, C.c_void_p, C.c_size_t, C.c_void_p]
+    lib.fl_prefill_mask_classify.restype = C.c_int
     lib.fl_rope_table.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_float, C.c_void_p]
     lib.fl_rope_table.restype = C.c_int
     lib.fl_attn_strerror.argtypes = [C.c_int]

@@ -335,7 +335,7 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
                           stream, p);
     if (e != hipSuccess) return e;
     const unsigned qblocks = (unsigned)((p.S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock);
-    if (p.attn_mask) {
+    if (p.attn_mask && !p.class_table) { // no table of the whole mask at hand: classify the rows of this call
         const int ktiles = (p.start_pos + p.S + flattn::kPrefillKeysPerStep - 1) / flattn::kPrefillKeysPerStep;
         e = launch(flattn::prefill_mask_classify_kernel, dim3((unsigned)ktiles, qblocks), dim3(256), stream, p, ktiles);
         if (e != hipSuccess) return e;
@@ -622,6 +622,10 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     p.k_cache = io->k_cache; p.v_cache = io->v_cache;
     p.freq_cis = io->freq_cis; p.attn_mask = io->attn_mask;
     p.tile_class = reinterpret_cast<uint32_t *>(ws + wl.tile_class);
+    if (io->mask_tile_classes && io->attn_mask && io->mask_ld >= L && io->start_pos % 32 == 0) {
+        p.class_table = static_cast<const uint8_t *>(io->mask_tile_classes);
+        p.class_ld = (L + 31) / 32;
+    }
     p.out = io->out ? io->out : reinterpret_cast<float *>(ws + wl.tmp_out);
     p.inp_scale = io->qkv_inp_scale; p.wq_scale = io->q_weight_scale;
     p.wk_scale = io->k_weight_scale; p.wv_scale = io->v_weight_scale;
@@ -639,6 +643,33 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
                               stream, p.out, io->out_int8, io->out_scale, desc->head_num, seq_len, D)))
             return FL_ATTN_ERR_HIP;
     }
+    return FL_ATTN_OK;
+}
+
+int fl_prefill_mask_classes_bytes(const fl_attn_desc *desc, size_t *bytes)
+{
+    if (!bytes) return FL_ATTN_ERR_NULL_POINTER;
+    int st = validate_desc(desc);
+    if (st != FL_ATTN_OK) return st;
+    const size_t n = ((size_t)desc->total_len + 31) / 32;
+    *bytes = n * n;
+    return FL_ATTN_OK;
+}
+
+int fl_prefill_mask_classify(const fl_attn_desc *desc, const float *attn_mask, int64_t mask_ld, void *classes,
+                             size_t classes_bytes, void *hip_stream)
+{
+    int st = validate_desc(desc);
+    if (st != FL_ATTN_OK) return st;
+    if (!attn_mask || !classes) return FL_ATTN_ERR_NULL_POINTER;
+    const int L = desc->total_len;
+    const size_t n = ((size_t)L + 31) / 32;
+    if (mask_ld < L) return FL_ATTN_ERR_ARGUMENT;
+    if (classes_bytes < n * n) return FL_ATTN_ERR_WORKSPACE;
+    if (n > 65535) return FL_ATTN_ERR_SHAPE;
+    if (!check_hip(launch(flattn::mask_class_table_kernel, dim3((unsigned)n, (unsigned)n), dim3(64), static_cast<hipStream_t>(hip_stream),
+                          attn_mask, mask_ld, L, L, static_cast<uint8_t *>(classes), (int)n)))
+        return FL_ATTN_ERR_HIP;
     return FL_ATTN_OK;
 }
 

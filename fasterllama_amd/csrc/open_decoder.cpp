@@ -82,7 +82,11 @@ namespace FasterLLaMA
         n += roundUp(tokens * sizeof(float), 256);
         n += 3 * roundUp(tokens * hidden_units_ * sizeof(int32_t), 256);
         n += roundUp(tokens * sizeof(float), 256);
-        return n + roundUp(decodeWorkspaceBytes(), 256) + roundUp(promptWorkspaceBytes(), 256) + 256; // slack to align a caller's base pointer
+        size_t classes = 0;
+        fl_attn_desc d = makeDesc<float>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
+        throwOnStatus(fl_prefill_mask_classes_bytes(&d, &classes), "getWorkspaceSize");
+        return n + roundUp(decodeWorkspaceBytes(), 256) + roundUp(promptWorkspaceBytes(), 256) + roundUp(classes, 256) +
+               256; // slack to align a caller's base pointer
     }
 
     template <OperationType OpType_, OperationType QuantizationType>
@@ -118,10 +122,27 @@ namespace FasterLLaMA
         p += roundUp(attn_workspace_bytes_, 256);
         prompt_workspace_ = p;
         prompt_workspace_bytes_ = promptWorkspaceBytes();
+        p += roundUp(prompt_workspace_bytes_, 256);
+        mask_classes_ = p;
+        mask_classified_ = false;
         // arrival counters of the decode scratch start at zero (a small kernel on the caller's stream); from
         // here on a decode step whose context is split is a single launch
         fl_attn_desc d = makeDesc<float>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
         throwOnStatus(fl_decode_attn_workspace_init(&d, attn_workspace_, attn_workspace_bytes_, param_.stream), "initialize");
+        throwOnStatus(fl_prefill_mask_classes_bytes(&d, &mask_classes_bytes_), "initialize");
+    }
+
+    template <OperationType OpType_, OperationType QuantizationType>
+    void OpenDecoder<OpType_, QuantizationType>::classifyMask()
+    {
+        if (!mask_classes_)
+            throw std::runtime_error("[FL][ERROR] classifyMask: initialize() has not been called");
+        mask_classified_ = false;
+        if (!param_.attn_mask) return;
+        fl_attn_desc d = makeDesc<float>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
+        throwOnStatus(fl_prefill_mask_classify(&d, param_.attn_mask, total_len_, mask_classes_, mask_classes_bytes_, param_.stream),
+                      "classifyMask");
+        mask_classified_ = true;
     }
 
     template <OperationType OpType_, OperationType QuantizationType>
@@ -147,6 +168,7 @@ namespace FasterLLaMA
         io.workspace = seq_len == 1 ? attn_workspace_ : prompt_workspace_;
         io.workspace_bytes = seq_len == 1 ? attn_workspace_bytes_ : prompt_workspace_bytes_;
         io.flags = seq_len == 1 ? FL_ATTN_IO_WORKSPACE_READY : 0;
+        io.mask_tile_classes = mask_classified_ ? mask_classes_ : nullptr;
         io.start_pos = start_pos;
         io.rope_row = literal_rope_row_ ? 0 : FL_ATTN_ROPE_AT_POSITION;
         io.max_start_pos = -1;

@@ -144,6 +144,9 @@ namespace FasterLLaMA
         size_t attn_workspace_bytes_ = 0;
         char *prompt_workspace_ = nullptr;        // scratch of the prompt-phase kernels
         size_t prompt_workspace_bytes_ = 0;
+        char *mask_classes_ = nullptr;            // tile classes of param_.attn_mask, see classifyMask()
+        size_t mask_classes_bytes_ = 0;
+        bool mask_classified_ = false;
 
         size_t decodeWorkspaceBytes() const;
         size_t promptWorkspaceBytes() const;
@@ -179,6 +182,10 @@ namespace FasterLLaMA
         void setExternalStages(const DecoderExternalStages<DataType_> &stages) { stages_ = stages; }
         void setLiteralRopeRow(bool literal) { literal_rope_row_ = literal; }
         void setContextSplits(int nsplit) { nsplit_ = nsplit; } // 0 = chosen by the library
+        // Classifies the tiles of param_.attn_mask once (on param_.stream), so that prompt-phase calls do not
+        // classify the rows they use on every call.  Call it after the mask has been filled, and again when its
+        // contents change; without it every prompt-phase call classifies for itself.
+        void classifyMask();
 
         // The attention segment alone on explicit operands: q/k/v are the float (or half, matching the
         // cache type) outputs of the projections, [B, 1, head_num, size_per_head]; attn_out is

@@ -30,7 +30,9 @@ struct PrefillParams {
     void *k_cache, *v_cache;       // [B,H,L,D]
     const float *freq_cis;
     const float *attn_mask;
-    uint32_t *tile_class; // workspace [ceil(S/128), ceil((start_pos+S)/32)]: mask tile classes (fp16 caches with a mask)
+    uint32_t *tile_class; // workspace [ceil(S/128), ceil((start_pos+S)/32)]: mask tile classes of this call, or
+    const uint8_t *class_table; // the caller's table over the whole mask (mask_class_table_kernel), row stride class_ld
+    int32_t class_ld;
     float *out;   // [B,H,S,D] fp32
     const float *inp_scale, *wq_scale, *wk_scale, *wv_scale;
     int64_t mask_ld;
@@ -122,6 +124,22 @@ constexpr int kPrefillQueriesPerBlock = 128; // 4 waves x 32 queries
 constexpr int kPrefillKeysPerStep = 32;
 constexpr uint32_t kTileSkip = 0, kTileZero = 1, kTileMixed = 2; // mask tile classes, see prefill_mask_classify_kernel
 
+// Classes of key tile t for the four 32-query sub-blocks of 128-query block qb, one per byte: from the words
+// this call's classify kernel wrote, or from the caller's persistent table over the whole mask (one byte per
+// 32-row block x 32-key tile, rows in blocks of 32 from mask row 0; start_pos is a multiple of 32 then).
+__device__ __forceinline__ uint32_t tile_class_word(const PrefillParams &p, int qb, int t, int NT)
+{
+    if (p.class_table) {
+        const uint8_t *row = p.class_table + (size_t)(p.start_pos / 32 + 4 * qb) * p.class_ld + t;
+        uint32_t w = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            if (qb * kPrefillQueriesPerBlock + 32 * k < p.S) w |= (uint32_t)row[(size_t)k * p.class_ld] << (8 * k);
+        return w; // sub-blocks beyond the prompt: kTileSkip
+    }
+    return p.tile_class[(size_t)qb * NT + t];
+}
+
 // Workgroup id -> (query block, head).  Consecutive ids go round-robin to the 8 XCDs, each with its
 // own L2, and every query block of a (b,h) reads that head's whole K and V: the blocks of one head
 // are therefore given consecutive slots of ONE XCD, so they run at the same time, walk the keys in
@@ -204,14 +222,14 @@ void prefill_attn_kernel(const PrefillParams p)
     // neither loaded nor multiplied, a wave skips the tiles it alone does not need, and the mask is
     // only read where it is not all zero.  Each of these leaves every bit of the result as it is:
     // the dropped terms are exp(v - max) == 0 and fma(s, scale, 0) == s*scale.
-    const uint32_t *cls = HAS_MASK ? p.tile_class + (size_t)qb * ((ctx + BN - 1) / BN) : nullptr;
-    uint32_t word_next = HAS_MASK ? cls[0] : 0u;
+    const int NTC = (ctx + BN - 1) / BN;
+    uint32_t word_next = HAS_MASK ? tile_class_word(p, qb, 0, NTC) : 0u;
 
     for (int k0 = 0; k0 < ctx; k0 += BN) {
         uint32_t tc = kTileZero;
         if constexpr (HAS_MASK) {
             const uint32_t word = __builtin_amdgcn_readfirstlane(word_next);
-            if (k0 + BN < ctx) word_next = cls[k0 / BN + 1]; // in flight during this tile
+            if (k0 + BN < ctx) word_next = tile_class_word(p, qb, k0 / BN + 1, NTC); // in flight during this tile
             if (word == 0u) continue;
             tc = (word >> (8 * wave)) & 0xffu;
         }
@@ -357,6 +375,27 @@ __global__ __launch_bounds__(256) void prefill_mask_classify_kernel(const Prefil
     if (tid == 0) p.tile_class[(size_t)qb * NT + t] = s_cls[0] | (s_cls[1] << 8) | (s_cls[2] << 16) | (s_cls[3] << 24);
 }
 
+// The same classes for a WHOLE mask [rows, cols] (row stride mask_ld), once per mask instead of once per call:
+// one byte per (32-row block, 32-key tile); entries past the last row / column repeat the last one.
+// grid = (ceil(cols/32), ceil(rows/32)), block = 64.
+__global__ __launch_bounds__(64) void mask_class_table_kernel(const float *mask, int64_t mask_ld, int rows, int cols,
+                                                              uint8_t *table, int table_ld)
+{
+    const int t = blockIdx.x, rb = blockIdx.y, lane = threadIdx.x;
+    const int col = min(t * kPrefillKeysPerStep + (lane & 31), cols - 1);
+    uint32_t nonzero = 0;
+    bool open = false;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int r = min(rb * 32 + 2 * j + (lane >> 5), rows - 1);
+        const float v = mask[(size_t)r * mask_ld + col];
+        nonzero |= __float_as_uint(v) << 1; // the sign is shifted out: -0 counts as zero
+        open |= !(v <= kMaskedBelow);       // a NaN entry keeps the tile
+    }
+    const uint32_t cls = __ballot(open) == 0ull ? kTileSkip : (__ballot(nonzero != 0u) == 0ull ? kTileZero : kTileMixed);
+    if (lane == 0) table[(size_t)rb * table_ld + t] = (uint8_t)cls;
+}
+
 // ---------------------------------------------------------------- fp16 caches: fp16 MFMA
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -468,7 +507,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         for (int base = c0; base < c1; base += 256) {
             const int t = base + tid;
             uint32_t w = 0;
-            if (t < c1) w = p.tile_class[(size_t)qb * NT + t];
+            if (t < c1) w = tile_class_word(p, qb, t, NT);
             const bool active = w != 0u;
             const unsigned long long bal = __ballot(active);
             if (lane == 0) s_wave_cnt[wave] = __popcll(bal);
@@ -875,13 +914,12 @@ __global__ __launch_bounds__(kWideWaves * 64) void prefill_attn_wide_kernel(cons
     const float scale = p.scale;
     const int NT = (ctx + BN - 1) / BN;
     // class of this 32-query block per key tile: byte (qb % 4) of the word of its 128-query block
-    const uint32_t *cls = HAS_MASK ? p.tile_class + (size_t)(qb / 4) * NT : nullptr;
 
     int buf = 0;
     for (int t = 0; t < NT; ++t) {
         uint32_t tc = kTileZero;
         if constexpr (HAS_MASK) {
-            tc = (__builtin_amdgcn_readfirstlane(cls[t]) >> (8 * (qb & 3))) & 0xffu;
+            tc = (__builtin_amdgcn_readfirstlane(tile_class_word(p, qb / 4, t, NT)) >> (8 * (qb & 3))) & 0xffu;
             if (tc == kTileSkip) continue; // uniform over the workgroup: every wave skips the same tiles
         }
         const int k0 = t * BN;

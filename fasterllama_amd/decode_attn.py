@@ -61,7 +61,7 @@ class DecodeAttention:
                 rope_row: int = capi.FL_ATTN_ROPE_AT_POSITION, attn_mask=None, mask_ld: int | None = None,
                 start_pos_per_seq=None, max_start_pos: int = -1, qkv_inp_scale=None,
                 q_weight_scale=None, k_weight_scale=None, v_weight_scale=None, out_int8=None,
-                out_scale=None) -> capi.AttnIO:
+                out_scale=None, mask_tile_classes=None) -> capi.AttnIO:
         io = capi.AttnIO()
         io.q, io.k_new, io.v_new = _ptr(q), _ptr(k_new), _ptr(v_new)
         io.k_cache, io.v_cache = _ptr(k_cache), _ptr(v_cache)
@@ -82,6 +82,7 @@ class DecodeAttention:
         io.v_weight_scale = _ptr(v_weight_scale)
         io.out_int8 = _ptr(out_int8)
         io.out_scale = _ptr(out_scale)
+        io.mask_tile_classes = _ptr(mask_tile_classes)
         return io
 
     def launch(self, io: capi.AttnIO, passes: int = 3, stream: torch.cuda.Stream | None = None) -> int:
@@ -127,6 +128,18 @@ class PrefillAttention(DecodeAttention):
         capi.check(self.lib.fl_prefill_attn_workspace_bytes(C.byref(self.desc), max_seq_len, C.byref(n)))
         self.max_seq_len = max_seq_len
         self.workspace = torch.empty(max(n.value, self.workspace.numel()), dtype=torch.uint8, device=self.device)
+
+    def classify_mask(self, attn_mask, mask_ld: int | None = None) -> torch.Tensor:
+        """fl_prefill_mask_classify: the tile classes of a whole [L, L] mask, to pass as mask_tile_classes."""
+        n = C.c_size_t(0)
+        capi.check(self.lib.fl_prefill_mask_classes_bytes(C.byref(self.desc), C.byref(n)))
+        table = torch.empty(n.value, dtype=torch.uint8, device=self.device)
+        s = torch.cuda.current_stream(self.device)
+        with torch.cuda.device(self.device):
+            capi.check(self.lib.fl_prefill_mask_classify(C.byref(self.desc), attn_mask.data_ptr(),
+                                                         self.desc.total_len if mask_ld is None else mask_ld,
+                                                         table.data_ptr(), table.numel(), C.c_void_p(s.cuda_stream)))
+        return table
 
     def launch_prefill(self, io: capi.AttnIO, seq_len: int, stream: torch.cuda.Stream | None = None) -> int:
         s = stream if stream is not None else torch.cuda.current_stream(self.device)

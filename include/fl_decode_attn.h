@@ -123,6 +123,9 @@ typedef struct fl_attn_io {
     /* optional epilogue: per-row absmax INT8 quantisation of out */
     int8_t *out_int8; /* [B, H*D] or NULL */
     float *out_scale; /* [B] (absmax/127), required with out_int8 */
+    /* optional, prompt phase: tile classes of the whole attn_mask from fl_prefill_mask_classify(), so that
+     * the mask is classified once per mask and not once per call (ignored by the decode step) */
+    const void *mask_tile_classes;
 } fl_attn_io;
 
 /* Launch plan the library would use for a context of ctx rows (ctx = start_pos + 1). */
@@ -194,6 +197,17 @@ int fl_decode_attn_forward_noalloc(const fl_attn_desc *desc, const fl_attn_io *i
 int fl_prefill_attn_workspace_bytes(const fl_attn_desc *desc, int32_t seq_len, size_t *bytes);
 int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int32_t seq_len,
                             void *hip_stream);
+
+/* The mask of the reference is one [L, L] array that every layer and every call reuses
+ * (samples/llama_fp16.cu:139-150), so its 32 x 32 tiles can be classified (all <= -1e30 / all zero / mixed)
+ * once: fl_prefill_mask_classify writes one byte per tile, ceil(L/32)^2 bytes (fl_prefill_mask_classes_bytes),
+ * for a mask with total_len rows and columns and row stride mask_ld >= total_len.  A prompt-phase call whose
+ * io.mask_tile_classes points at that table, with the same attn_mask and mask_ld and a start_pos that is a
+ * multiple of 32, skips its own classification launch; any other call classifies the rows it uses as before.
+ * The table is valid until the mask's contents change. */
+int fl_prefill_mask_classes_bytes(const fl_attn_desc *desc, size_t *bytes);
+int fl_prefill_mask_classify(const fl_attn_desc *desc, const float *attn_mask, int64_t mask_ld, void *classes,
+                             size_t classes_bytes, void *hip_stream);
 
 /* RoPE table producer on the device: rows x D floats, row r = [cos(r*w_0), sin(r*w_0), ...],
  * w_i = base^(-2i/D).  Replaces launchPrecomputeFreqsCis (decoding_kernels.cu:85-135,

@@ -257,6 +257,7 @@ template <OperationType Op, typename CacheT> static void runAll(const char *tag)
         st2.post_attention = postHook<DataT>;
         dec.setExternalStages(st2);
         DevBuf<DataT> d_from((size_t)B * S * HD), d_dec_out((size_t)B * S * HD);
+        dec.classifyMask(); // the mask is in place: its tiles are classified once, not in every prompt-phase call
         dec.forward(d_from.p, d_freq.p, d_kc.p, d_vc.p, d_dec_out.p, 0, S);
         HIP_OK(hipStreamSynchronize(stream));
 

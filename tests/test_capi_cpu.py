@@ -39,9 +39,9 @@ def test_header_and_binding_agree_and_library_exports_everything():
 
 
 def test_struct_layouts_match_the_header():
-    # natural alignment on x86-64: 8 x 4 bytes, and 10 pointers/size_t + int64 + 4 x int32 + 6 pointers
+    # natural alignment on x86-64: 8 x 4 bytes, and 10 pointers/size_t + int64 + 4 x int32 + 7 pointers
     assert C.sizeof(capi.AttnDesc) == 32
-    assert C.sizeof(capi.AttnIO) == 10 * 8 + 8 + 8 + 16 + 6 * 8
+    assert C.sizeof(capi.AttnIO) == 10 * 8 + 8 + 8 + 16 + 7 * 8
     assert C.sizeof(capi.AttnPlan) == 16
 
 

@@ -372,6 +372,45 @@ def test_prefill_int32_prologue_and_int8_epilogue(gpu):
     assert np.abs(q8.cpu().numpy().astype(np.int32) - q_or.astype(np.int32)).max() <= 1
 
 
+@pytest.mark.parametrize("dtype,D", [("f16", 128), ("f32", 128), ("f16", 64), ("f16", 256), ("f32", 512)])
+def test_prefill_with_a_persistent_mask_class_table(gpu, dtype, D):
+    """fl_prefill_mask_classify once per mask instead of a classification launch per call: bit-identical outputs
+    for masks with dropped, zero and mixed tiles, at start positions that use the table (multiples of 32) and
+    at one that falls back to the per-call classification."""
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    B, H, L = 2, 3, 320
+    tdt = torch.float16 if dtype == "f16" else torch.float32
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+    r, c = np.arange(L)[:, None], np.arange(L)[None, :]
+    masks = {
+        "causal -FLT_MAX": np.where(c > r, -FMAX, 0.0),
+        "causal -1e5": np.where(c > r, -1e5, 0.0),
+        "window 70": np.where((c > r) | (c < r - 70), -FMAX, 0.0),
+        "dense random": np.random.default_rng(4).standard_normal((L, L)) * 2,
+    }
+    for name, m in masks.items():
+        m = m.astype(np.float32)
+        for S, P in ((100, 0), (129, 64), (60, 224), (50, 37)):
+            q, k, v, kc, vc, f = make(B, H, D, L, S, dtype, 7 + S)
+            want = ref.prefill_attn(q, k, v, kc.copy(), vc.copy(), f, start_pos=P, attn_mask=m, acc_double=True, threads=16)
+            op = PrefillAttention(B, H, D, L, S, tdt, device=gpu)
+            md = t(m)
+            table = op.classify_mask(md)
+            outs = []
+            for tab in (None, table):
+                kc_d, vc_d = t(kc), t(vc)
+                outs.append(op.prefill(t(q), t(k), t(v), kc_d, vc_d, t(f), start_pos=P, attn_mask=md,
+                                       mask_tile_classes=tab).cpu().numpy())
+            assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32)), f"{name} S={S} P={P}"
+            assert_out_close(outs[1], want, dtype, f"class table, {name} S={S} P={P}",
+                             float_ref=lambda: ref.prefill_attn(q, k, v, kc.copy(), vc.copy(), f, start_pos=P, attn_mask=m, threads=16))
+    # the table itself: 0 = every entry <= -1e30, 1 = every entry zero, 2 = anything else
+    tab = op.classify_mask(t(masks["causal -FLT_MAX"].astype(np.float32))).cpu().numpy().reshape(10, 10)
+    assert (np.diag(tab) == 2).all() and (np.tril(tab, -1)[np.tril_indices(10, -1)] == 1).all() \
+        and (tab[np.triu_indices(10, 1)] == 0).all()
+
+
 def test_prefill_argument_errors(gpu):
     import torch
     from fasterllama_amd.decode_attn import PrefillAttention
