@@ -96,8 +96,23 @@ def bench_prefill(args) -> int:
     table = None
     if args.prefill_mask != "none" and not args.prefill_classify_per_call:
         table = op.classify_mask(mask)
+    extra = {}
+    if args.segment == "int32-int8":
+        # the segment as OpenDecoder::forward feeds it: int32 accumulators + scales in, per-token INT8 + scale out, no
+        # float output (the float result passes through the workspace to the quantisation kernel)
+        args.no_cpu = True
+        rng = np.random.default_rng(args.seed)
+        q, k, v = (torch.from_numpy(rng.integers(-20000, 20000, (B, S, H, D), dtype=np.int32)).to(dev) for _ in range(3))
+        extra = dict(
+            qkv_inp_scale=torch.from_numpy(((rng.random(B * S) + 0.5) * 2e-3).astype(np.float32)).to(dev),
+            q_weight_scale=torch.from_numpy((rng.random(H * D) * 3e-2 + 1e-3).astype(np.float32)).to(dev),
+            k_weight_scale=torch.from_numpy((rng.random(H * D) * 3e-2 + 1e-3).astype(np.float32)).to(dev),
+            v_weight_scale=torch.from_numpy((rng.random(H * D) * 3e-2 + 1e-3).astype(np.float32)).to(dev),
+            out_int8=torch.empty(B, S, H * D, dtype=torch.int8, device=dev),
+            out_scale=torch.empty(B, S, dtype=torch.float32, device=dev))
+        out = None
     io = op.make_io(q, k, v, kc, vc, freq, out, start_pos=P, attn_mask=None if args.prefill_mask == "none" else mask,
-                    mask_tile_classes=table)
+                    mask_tile_classes=table, **extra)
     stream = torch.cuda.current_stream(dev)
 
     def run(n):
@@ -153,7 +168,8 @@ def bench_prefill(args) -> int:
                                   "block-causal": "additive mask, causal over blocks of 128 tokens, -FLT_MAX above",
                                   "none": "no mask"}[args.prefill_mask]
                                + (", fast first product (fp16 queries)" if args.prefill_fast_qk and w["dtype"] == "f16" else "")
-                               + (", mask tiles classified once per mask" if table is not None else ""),
+                               + (", mask tiles classified once per mask" if table is not None else "")
+                               + (", int32 accumulators in, INT8 + scale out" if args.segment == "int32-int8" else ""),
                    "flops_per_step": flops, "dense_flops_per_step": dense_flops,
                    "tokens_per_s": round(B * S / (ms * 1e-3), 1)},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": peak, "unit": "TFLOP/s",

@@ -450,6 +450,7 @@ int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_str
     const bool quant = io->out_int8 != nullptr;
     if (!io->out && !quant) return FL_ATTN_ERR_NULL_POINTER;
     if (quant && !io->out_scale) return FL_ATTN_ERR_NULL_POINTER;
+    if (quant && (reinterpret_cast<uintptr_t>(io->out_int8) & 3u) != 0) return FL_ATTN_ERR_ALIGNMENT; // written four at a time
     if ((io->flags & ~FL_ATTN_IO_WORKSPACE_READY) != 0) return FL_ATTN_ERR_ARGUMENT;
     const bool i32 = io->qkv_inp_scale != nullptr;
     if (i32 && (!io->q_weight_scale || !io->k_weight_scale || !io->v_weight_scale)) return FL_ATTN_ERR_NULL_POINTER;
@@ -596,6 +597,7 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     const bool quant = io->out_int8 != nullptr;
     if (!io->out && !quant) return FL_ATTN_ERR_NULL_POINTER;
     if (quant && !io->out_scale) return FL_ATTN_ERR_NULL_POINTER;
+    if (quant && (reinterpret_cast<uintptr_t>(io->out_int8) & 3u) != 0) return FL_ATTN_ERR_ALIGNMENT; // written four at a time
     if (io->flags != 0 || io->start_pos_per_seq) return FL_ATTN_ERR_ARGUMENT; // uniform positions only
     const bool i32 = io->qkv_inp_scale != nullptr;
     if (i32 && (!io->q_weight_scale || !io->k_weight_scale || !io->v_weight_scale)) return FL_ATTN_ERR_NULL_POINTER;

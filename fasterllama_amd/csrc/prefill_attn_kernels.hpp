@@ -1032,8 +1032,25 @@ __global__ __launch_bounds__(1024) void attn_quantize_transpose_kernel(const flo
     const int b = bs / S, s = bs % S;
     const int HD = H * D;
     const float *x = attn + ((size_t)b * H * S + s) * D; // + h * S * D + d
+    // A token of up to 8192 values is read ONCE, four consecutive values per lane and trip, and stays in
+    // registers between the absmax reduction and the rounding; longer tokens are read twice.
+    constexpr int KEEP = 2; // float4 per thread held in registers
+    const bool keep = HD <= 1024 * 4 * KEEP && (D & 3) == 0;
+    float4 held[KEEP];
     float absmax = kMaxFloor;
-    for (int e = tid; e < HD; e += 1024) absmax = fmaxf(absmax, fabsf(x[(size_t)(e / D) * S * D + e % D]));
+    if (keep) {
+#pragma unroll
+        for (int k = 0; k < KEEP; ++k) {
+            const int e = (tid + k * 1024) * 4;
+            held[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (e < HD) {
+                held[k] = *reinterpret_cast<const float4 *>(x + (size_t)(e / D) * S * D + e % D);
+                absmax = fmaxf(fmaxf(absmax, fmaxf(fabsf(held[k].x), fabsf(held[k].y))), fmaxf(fabsf(held[k].z), fabsf(held[k].w)));
+            }
+        }
+    } else {
+        for (int e = tid; e < HD; e += 1024) absmax = fmaxf(absmax, fabsf(x[(size_t)(e / D) * S * D + e % D]));
+    }
     absmax = wave_max(absmax);
     if ((tid & 63) == 0) s_red[tid >> 6] = absmax;
     __syncthreads();
@@ -1041,10 +1058,23 @@ __global__ __launch_bounds__(1024) void attn_quantize_transpose_kernel(const flo
 #pragma unroll
     for (int w = 1; w < 16; ++w) absmax = fmaxf(absmax, s_red[w]);
     if (tid == 0) out_scale[bs] = absmax / 127.0f;
-    for (int e = tid; e < HD; e += 1024) {
-        const float v = rintf(__fmul_rn(x[(size_t)(e / D) * S * D + e % D], 127.0f) / absmax);
-        const int qv = (v != v) ? 0 : (int)fminf(fmaxf(v, -128.f), 127.f); // NaN -> 0, saturate
-        out_q[(size_t)bs * HD + e] = (int8_t)qv;
+    auto quant = [&](float value) -> int {
+        const float v = rintf(__fmul_rn(value, 127.0f) / absmax);
+        return (v != v) ? 0 : (int)fminf(fmaxf(v, -128.f), 127.f); // NaN -> 0, saturate
+    };
+    if (keep) {
+#pragma unroll
+        for (int k = 0; k < KEEP; ++k) {
+            const int e = (tid + k * 1024) * 4;
+            if (e < HD) {
+                const uint32_t packed = (uint32_t)(quant(held[k].x) & 0xff) | (uint32_t)(quant(held[k].y) & 0xff) << 8 |
+                                        (uint32_t)(quant(held[k].z) & 0xff) << 16 | (uint32_t)(quant(held[k].w) & 0xff) << 24;
+                *reinterpret_cast<uint32_t *>(out_q + (size_t)bs * HD + e) = packed;
+            }
+        }
+    } else {
+        for (int e = tid; e < HD; e += 1024)
+            out_q[(size_t)bs * HD + e] = (int8_t)quant(x[(size_t)(e / D) * S * D + e % D]);
     }
 }
 

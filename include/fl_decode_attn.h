@@ -121,7 +121,7 @@ typedef struct fl_attn_io {
     const float *k_weight_scale; /* [H*D] */
     const float *v_weight_scale; /* [H*D] */
     /* optional epilogue: per-row absmax INT8 quantisation of out */
-    int8_t *out_int8; /* [B, H*D] or NULL */
+    int8_t *out_int8; /* [B, H*D] or NULL; 4-byte aligned */
     float *out_scale; /* [B] (absmax/127), required with out_int8 */
     /* optional, prompt phase: tile classes of the whole attn_mask from fl_prefill_mask_classify(), so that
      * the mask is classified once per mask and not once per call (ignored by the decode step) */
