@@ -151,7 +151,7 @@ def test_prefill_small_heads_with_causal_mask(gpu, dtype, D):
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
 def test_prefill_sharp_softmax_with_scaled_keys(gpu, dtype):
-    """Some key rows scaled by 8 (the stress of BASELINE configuration 4): near one-hot weights, running maxima
+    """Some key rows scaled by 8 (the stress of the B=1, ctx=4096 benchmark configuration): near one-hot weights, running maxima
     that jump late in the walk over the keys, and scores far above the lazily updated reference maximum."""
     import torch
     from fasterllama_amd.decode_attn import PrefillAttention
