@@ -468,8 +468,15 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     constexpr bool PF_KA = HAS_MASK || QSPLIT;
     constexpr bool PF_VA = HAS_MASK && !QSPLIT;
     constexpr int BN = kPrefillKeysPerStep; // 32
-    constexpr int LDK = D + 8;              // halfs; rows start 4 banks apart (128-bit operand reads)
-    constexpr int LDV = D + 32;             // halfs; rows start 16 banks apart (8 rows x 64 bytes per transposing read)
+    // D = 128: the key tiles go from global memory STRAIGHT into LDS (buffer_load ... lds, 16 bytes per lane): no
+    // staging registers, no ds_write, no wait for a load in the middle of the loop.  Such a load lays the 64 lanes'
+    // chunks down back to back (1 KB = four 256-byte rows), so rows cannot be padded against bank conflicts;
+    // the tiles are swizzled instead — row r keeps its 16-byte chunk c of K at position c ^ (r & 15), and its
+    // 32-byte unit u of V at position u ^ (r & 7) — which each lane applies to the GLOBAL address it loads from.
+    constexpr bool DMA = D == 128;
+    constexpr int NBUF = DMA ? 3 : 2;       // tile buffers: a direct load is issued two tiles ahead
+    constexpr int LDK = DMA ? D : D + 8;    // halfs; padded rows start 4 banks apart (128-bit operand reads)
+    constexpr int LDV = DMA ? D : D + 32;   // halfs; padded rows start 16 banks apart (8 rows x 64 bytes per transposing read)
     constexpr int NC = D / 16;
     constexpr int NDT = D / 32;
     constexpr int CPR = D / 8; // 16-byte chunks per cache row
@@ -479,13 +486,20 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     constexpr int LDQ = D + 8;              // halfs; the workgroup's rotated queries pass through the tile buffers once
     constexpr int HALF_D = D >= 128 ? 64 : 32; // output columns per epilogue pass
     constexpr int LDO = HALF_D + 4;         // floats; the output block passes through the tile buffers too
-    constexpr int TILE_HALFS = 2 * BN * (LDK + LDV), Q_HALFS = kPrefillQueriesPerBlock * LDQ,
+    constexpr int TILE_HALFS = NBUF * BN * (LDK + LDV), Q_HALFS = kPrefillQueriesPerBlock * LDQ,
                   O_HALFS = kPrefillQueriesPerBlock * LDO * 2;
-    constexpr int SMEM_HALFS = TILE_HALFS > Q_HALFS ? (TILE_HALFS > O_HALFS ? TILE_HALFS : O_HALFS)
-                                                    : (Q_HALFS > O_HALFS ? Q_HALFS : O_HALFS);
+    // Padded layout: K tiles, then V tiles; the queries pass through the same bytes before the first tile is
+    // stored.  Swizzled layout: tile buffer b = K (8 KB) then V (8 KB) at b * 16 KB, and the queries pass through
+    // the bytes BEHIND buffer 0, so that the first tile can be requested before the queries are.
+    constexpr int Q_OFF = DMA ? BN * (LDK + LDV) : 0; // halfs
+    constexpr int Q_END = Q_OFF + Q_HALFS;
+    constexpr int SMEM_HALFS = TILE_HALFS > Q_END ? (TILE_HALFS > O_HALFS ? TILE_HALFS : O_HALFS)
+                                                  : (Q_END > O_HALFS ? Q_END : O_HALFS);
     __shared__ __attribute__((aligned(16))) _Float16 smem[SMEM_HALFS];
-    _Float16 (*sK)[BN][LDK] = reinterpret_cast<_Float16 (*)[BN][LDK]>(smem);
-    _Float16 (*sV)[BN][LDV] = reinterpret_cast<_Float16 (*)[BN][LDV]>(smem + 2 * BN * LDK);
+    _Float16 *const sQ = smem + Q_OFF;
+    _Float16 (*sK)[BN][LDK] = reinterpret_cast<_Float16 (*)[BN][LDK]>(smem);                   // padded layout only
+    _Float16 (*sV)[BN][LDV] = reinterpret_cast<_Float16 (*)[BN][LDV]>(smem + NBUF * BN * LDK); // padded layout only
+    constexpr uint32_t kTileBytes = (uint32_t)(BN * (LDK + LDV) * 2), kVOff = (uint32_t)(BN * LDK * 2); // swizzled layout
     __shared__ uint32_t s_list[HAS_MASK ? kTileListCap : 1];
     __shared__ int s_wave_cnt[4];
 
@@ -502,12 +516,14 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     // The tiles of [c0, c1) that some wave of this workgroup needs, in order, as a list in LDS:
     // entry = tile << 8 | the four waves' classes (2 bits each).  Built once per chunk of
     // kTileListCap tiles, so the loop below never chases a class word through memory.
-    auto build_list = [&](int c0, int c1) -> int {
+    // (w_first: this thread's class word of tile c0 + tid where the caller has loaded it already)
+    auto build_list = [&](int c0, int c1, bool have_first, uint32_t w_first) -> int {
         int count = 0;
         for (int base = c0; base < c1; base += 256) {
             const int t = base + tid;
             uint32_t w = 0;
-            if (t < c1) w = tile_class_word(p, qb, t, NT);
+            if (have_first && base == c0) w = w_first;
+            else if (t < c1) w = tile_class_word(p, qb, t, NT);
             const bool active = w != 0u;
             const unsigned long long bal = __ballot(active);
             if (lane == 0) s_wave_cnt[wave] = __popcll(bal);
@@ -547,7 +563,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         const int r = idx / CPR, cc = idx % CPR;
         src_off[j] = (EXACT || idx < BN * CPR) ? (uint32_t)(r * D * 2 + cc * 16) : kLaneOutOfRange;
         k_dst[j] = (uint32_t)((r * LDK + cc * 8) * 2);
-        v_dst[j] = (uint32_t)((2 * BN * LDK + r * LDV + cc * 8) * 2);
+        v_dst[j] = (uint32_t)((NBUF * BN * LDK + r * LDV + cc * 8) * 2);
     }
     auto fetch = [&](int t) {
         const uint32_t slab = (uint32_t)t * (uint32_t)(BN * D * 2); // uniform; part of the checked offset
@@ -568,12 +584,69 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         }
     };
 
-    // The list of the first chunk and its first tile are requested BEFORE the queries: the class words, the
-    // first K/V tile and the queries then travel together instead of one memory round trip after the other.
+    // Direct path.  One instruction moves 1 KB, four rows: lane -> row lane/16, 16-byte position lane%16.  Wave w
+    // issues the blocks 2w and 2w+1 of K and of V.  The range check of the descriptor (rows at or beyond the
+    // context arrive as zeros) applies to the lane offset only, so the tile's slab is added to it.
+    uint32_t dk_off[DMA ? 2 : 1], dv_off[DMA ? 2 : 1];
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    if constexpr (DMA) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int r = 8 * wave + 4 * j + (lane >> 4), pc = lane & 15;
+            dk_off[j] = (uint32_t)(r * 256 + ((pc ^ (r & 15)) << 4));
+            dv_off[j] = (uint32_t)(r * 256 + ((((pc >> 2) ^ (r & 3)) << 2 | (pc & 3)) << 4));
+        }
+    }
+    // The loads are written as assembly on purpose.  The compiler treats a direct load as a store to LDS that
+    // any later LDS read may alias, and as pending work every workgroup barrier must drain: it would put
+    // `s_waitcnt vmcnt(0)` before the transposing reads and before each barrier, which waits for the tile that
+    // was requested a moment ago and serialises the pipeline.  The loop below waits for exactly the tile it is
+    // about to read (s_waitcnt vmcnt(4): the newer tile's four loads may stay in flight) before its barrier.
+    // M0 carries the LDS address of the block; one wait state separates its write from the load that uses it.
+    typedef int int4v __attribute__((ext_vector_type(4)));
+    auto raw_descriptor = [&](const _Float16 *base) -> int4v {
+        const uint64_t a = reinterpret_cast<uint64_t>(base);
+        return int4v{(int)(uint32_t)a, (int)(uint32_t)(a >> 32), (int)((uint32_t)ctx * (uint32_t)(D * 2)), 0x00020000};
+    };
+    const int4v Kdesc = raw_descriptor(Kb), Vdesc = raw_descriptor(Vb);
+    typedef __attribute__((address_space(3))) _Float16 *lds_half_ptr;
+    const uint32_t lds_tiles = (uint32_t)(uintptr_t)(lds_half_ptr)smem + (uint32_t)wave_u * 2048u; // this wave's blocks
+    auto dma = [&](int t, int buf) {
+        const uint32_t slab = (uint32_t)t * (uint32_t)(BN * D * 2);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t k_lds = lds_tiles + (uint32_t)buf * kTileBytes + (uint32_t)(j * 1024);
+            const uint32_t v_lds = k_lds + kVOff;
+            uint32_t m0_saved; // M0 is the compiler's to use elsewhere: hand it back as it was
+            asm volatile("s_mov_b32 %0, m0\n\t"
+                         "s_mov_b32 m0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, 0 offen lds\n\t"
+                         "s_mov_b32 m0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %5, %6, 0 offen lds\n\t"
+                         "s_mov_b32 m0, %0"
+                         : "=&s"(m0_saved)
+                         : "s"(k_lds), "v"(dk_off[DMA ? j : 0] + slab), "s"(Kdesc), "s"(v_lds), "v"(dv_off[DMA ? j : 0] + slab), "s"(Vdesc)
+                         : "memory");
+        }
+    };
+    // LDS addresses of the operands.  Padded layout: plain rows.  Swizzled layout: K chunk 2c+hf of row qi sits
+    // at chunk (2c+hf) ^ (qi & 15) — one XOR with a constant per read — and the 64-byte unit dt of a V row at
+    // unit dt ^ (row & 3); the rows a lane reads differ by multiples of 8, which leaves row & 3 alone.
+    const uint32_t k_swz = (uint32_t)(qi * 256 + (((2 * 0 + hf) ^ (qi & 15)) << 4));
+    auto k_operand = [&](int buf, int c) -> half8 {
+        if constexpr (DMA) return *reinterpret_cast<const half8 *>(reinterpret_cast<const char *>(smem) + (uint32_t)buf * kTileBytes + (k_swz ^ (uint32_t)(c << 5)));
+        else return *reinterpret_cast<const half8 *>(&sK[buf][qi][16 * c + 8 * hf]);
+    };
+
+    // The class words of the first chunk, key tile 0 and the queries are requested together, so that they
+    // travel at the same time instead of one memory round trip after the other.  Tile 0 is a guess at the first
+    // listed tile (right without a mask and under every causal mask); the list is built after the queries are
+    // in, and a workgroup whose list starts elsewhere requests that tile then.
     const int first_c1 = min(kTileListCap, NT);
-    int n_first = first_c1;
-    if constexpr (HAS_MASK) n_first = build_list(0, first_c1);
-    if (n_first > 0) fetch((int)(__builtin_amdgcn_readfirstlane(list_entry(0, 0)) >> 8));
+    if constexpr (DMA) dma(0, 0);
+    else fetch(0);
+    uint32_t w_first = 0;
+    if constexpr (HAS_MASK) {
+        if (tid < first_c1) w_first = tile_class_word(p, qb, tid, NT);
+    }
 
     // Rotated queries of the workgroup: loaded and rotated cooperatively (16 lanes per 256-byte row, so
     // the [B,S,H,D] rows are read whole), rounded once to fp16 as MFMA operands, and handed to their
@@ -612,26 +685,40 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 hq[i] = valid ? (_Float16)x[j][i] : (_Float16)0;
                 if constexpr (QSPLIT) lo_keep[j][i] = valid ? (_Float16)(x[j][i] - (float)hq[i]) : (_Float16)0;
             }
-            *reinterpret_cast<half8 *>(smem + r * LDQ + cc * 8) = hq;
+            *reinterpret_cast<half8 *>(sQ + r * LDQ + cc * 8) = hq;
         }
         __syncthreads();
 #pragma unroll
         for (int c = 0; c < NC; ++c)
-            qreg[c] = *reinterpret_cast<const half8 *>(smem + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
+            qreg[c] = *reinterpret_cast<const half8 *>(sQ + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
         __syncthreads();
         if constexpr (QSPLIT) {
 #pragma unroll
             for (int j = 0; j < QPT; ++j) {
                 const int idx = tid + j * 256;
-                *reinterpret_cast<half8 *>(smem + (idx / CPR) * LDQ + (idx % CPR) * 8) = lo_keep[j];
+                *reinterpret_cast<half8 *>(sQ + (idx / CPR) * LDQ + (idx % CPR) * 8) = lo_keep[j];
             }
             __syncthreads();
 #pragma unroll
             for (int c = 0; c < NC; ++c)
-                qlo[c] = *reinterpret_cast<const half8 *>(smem + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
+                qlo[c] = *reinterpret_cast<const half8 *>(sQ + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
             __syncthreads();
         }
-        // the tile buffers are free for K and V
+        // the tile buffers behind the first are free for K and V
+    }
+    int n_first = first_c1;
+    if constexpr (HAS_MASK) n_first = build_list(0, first_c1, true, w_first);
+    if (n_first > 0) {
+        const int t_first = (int)(__builtin_amdgcn_readfirstlane(list_entry(0, 0)) >> 8);
+        if (t_first != 0) {
+            if constexpr (DMA) { // the guessed tile must have landed, in every wave, before its buffer is written again
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                dma(t_first, 0);
+            } else {
+                fetch(t_first);
+            }
+        }
     }
 
     floatx16 ot[NDT];
@@ -643,6 +730,11 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     float m = kMaxFloor * kLog2e, l = 0.f;
     // per-lane source of the transposing V reads: row 4hf + (lane%16)/4, halfs 16*((lane/16)%2) + 4*(lane%4)
     const int vrow = 4 * hf + ((lane & 15) >> 2), vcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    const uint32_t v_swz = (uint32_t)(vrow * 256 + ((vrow & 3) << 6) + vcol * 2);
+    auto v_operand = [&](int buf, int row0, int dt) -> half4 { // row0: 16u or 16u + 8
+        if constexpr (DMA) return lds_read_tr16(reinterpret_cast<const _Float16 *>(reinterpret_cast<const char *>(smem) + (uint32_t)buf * kTileBytes + kVOff + (uint32_t)(row0 * 256) + (v_swz ^ (uint32_t)(dt << 6))));
+        else return lds_read_tr16(&sV[buf][row0 + vrow][32 * dt + vcol]);
+    };
     const float inv_scale = 1.0f / p.scale;
     const bool mask_vec4 = HAS_MASK && (p.mask_ld & 3) == 0 && (reinterpret_cast<uintptr_t>(p.attn_mask) & 15u) == 0;
 
@@ -657,23 +749,32 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     for (int c0 = 0; c0 < NT; c0 += kTileListCap) {
         const int c1 = min(c0 + kTileListCap, NT);
         int n = c1 - c0;
-        if (c0 == 0) n = n_first; // built, and its first tile requested, before the queries were loaded
-        else if constexpr (HAS_MASK) n = build_list(c0, c1); // ends with a barrier: the tile buffers are free again
+        if (c0 == 0) n = n_first; // built, and its first tile requested, in the prologue
+        else if constexpr (HAS_MASK) n = build_list(c0, c1, false, 0u); // ends with a barrier: the tile buffers are free again
         else __syncthreads();
         if (n == 0) continue;
         uint32_t e0 = __builtin_amdgcn_readfirstlane(list_entry(c0, 0));
         uint32_t e1 = n > 1 ? __builtin_amdgcn_readfirstlane(list_entry(c0, 1)) : 0u;
         uint32_t e2 = n > 2 ? __builtin_amdgcn_readfirstlane(list_entry(c0, 2)) : 0u;
         uint32_t e3 = n > 3 ? list_entry(c0, 3) : 0u;
-        if (c0 > 0) fetch((int)(e0 >> 8));
-        commit(0);
-        if (n > 1) fetch((int)(e1 >> 8));
+        if constexpr (DMA) {
+            if (c0 > 0) dma((int)(e0 >> 8), 0);
+            if (n > 1) dma((int)(e1 >> 8), 1);
+        } else {
+            if (c0 > 0) fetch((int)(e0 >> 8));
+            commit(0);
+            if (n > 1) fetch((int)(e1 >> 8));
+        }
         // one tile of the pipeline; the LDS buffer index is a compile-time constant (the loop below is
         // unrolled by two), so every LDS address is a register plus an immediate
         auto tile_step = [&](int i, auto buf_tag) {
             constexpr int buf = decltype(buf_tag)::value;
             const int t = (int)(e0 >> 8);
-            __syncthreads(); // tile t is visible; every wave is done with the other buffer
+            if constexpr (DMA) { // this wave's part of tile t has landed; tile t+1 (four loads) may still be in flight
+                if (i + 1 < n) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+            __syncthreads(); // tile t is visible; every wave is done with the previous tile's buffer
 
             // The additive term enters as the initial value of the score accumulator, in units of the
             // raw product: (s + mask/scale)*scale.  Zero for most tiles; the mask entries where the tile
@@ -708,7 +809,9 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 }
             }
 
-            if (i + 1 < n) {
+            if constexpr (DMA) {
+                if (i + 2 < n) dma((int)(e2 >> 8), (buf + 2) % NBUF); // the buffer of tile t-1
+            } else if (i + 1 < n) {
                 commit(buf ^ 1);
                 if (i + 2 < n) fetch((int)(e2 >> 8));
             }
@@ -717,10 +820,10 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 half8 kall[PF_KA ? NC : 1];
                 if constexpr (PF_KA) {
 #pragma unroll
-                    for (int c = 0; c < NC; ++c) kall[c] = *reinterpret_cast<const half8 *>(&sK[buf][qi][16 * c + 8 * hf]);
+                    for (int c = 0; c < NC; ++c) kall[c] = k_operand(buf, c);
                     __builtin_amdgcn_sched_barrier(0);
                 } else {
-                    kall[0] = *reinterpret_cast<const half8 *>(&sK[buf][qi][8 * hf]);
+                    kall[0] = k_operand(buf, 0);
                 }
                 const half8 ka0 = kall[0];
                 if (special) {
@@ -742,7 +845,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 if constexpr (QSPLIT) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka0, qlo[0], st, 0, 0, 0);
 #pragma unroll
                 for (int c = 1; c < NC; ++c) {
-                    const half8 ka = PF_KA ? kall[PF_KA ? c : 0] : *reinterpret_cast<const half8 *>(&sK[buf][qi][16 * c + 8 * hf]);
+                    const half8 ka = PF_KA ? kall[PF_KA ? c : 0] : k_operand(buf, c);
                     st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[c], st, 0, 0, 0);
                     if constexpr (QSPLIT) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qlo[c], st, 0, 0, 0);
                 }
@@ -753,8 +856,8 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                     for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                         for (int u = 0; u < 2; ++u) {
-                            vlo[dt][u] = lds_read_tr16(&sV[buf][16 * u + vrow][32 * dt + vcol]);
-                            vhi[dt][u] = lds_read_tr16(&sV[buf][16 * u + 8 + vrow][32 * dt + vcol]);
+                            vlo[dt][u] = v_operand(buf, 16 * u, dt);
+                            vhi[dt][u] = v_operand(buf, 16 * u + 8, dt);
                         }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -791,8 +894,8 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
                     for (int u = 0; u < 2; ++u) {
-                        const half4 lo = PF_VA ? vlo[PF_VA ? dt : 0][u] : lds_read_tr16(&sV[buf][16 * u + vrow][32 * dt + vcol]);
-                        const half4 hi = PF_VA ? vhi[PF_VA ? dt : 0][u] : lds_read_tr16(&sV[buf][16 * u + 8 + vrow][32 * dt + vcol]);
+                        const half4 lo = PF_VA ? vlo[PF_VA ? dt : 0][u] : v_operand(buf, 16 * u, dt);
+                        const half4 hi = PF_VA ? vhi[PF_VA ? dt : 0][u] : v_operand(buf, 16 * u + 8, dt);
                         half8 va;
                         va[0] = lo[0]; va[1] = lo[1]; va[2] = lo[2]; va[3] = lo[3];
                         va[4] = hi[0]; va[5] = hi[1]; va[6] = hi[2]; va[7] = hi[3];
@@ -805,9 +908,17 @@ void prefill_attn_f16_kernel(const PrefillParams p)
             e2 = __builtin_amdgcn_readfirstlane(e3);
             e3 = i + 4 < n ? list_entry(c0, i + 4) : 0u;
         };
-        for (int i = 0; i < n; i += 2) {
-            tile_step(i, std::integral_constant<int, 0>{});
-            if (i + 1 < n) tile_step(i + 1, std::integral_constant<int, 1>{});
+        if constexpr (DMA) {
+            for (int i = 0; i < n; i += 3) {
+                tile_step(i, std::integral_constant<int, 0>{});
+                if (i + 1 < n) tile_step(i + 1, std::integral_constant<int, 1>{});
+                if (i + 2 < n) tile_step(i + 2, std::integral_constant<int, 2>{});
+            }
+        } else {
+            for (int i = 0; i < n; i += 2) {
+                tile_step(i, std::integral_constant<int, 0>{});
+                if (i + 1 < n) tile_step(i + 1, std::integral_constant<int, 1>{});
+            }
         }
     }
 
@@ -818,6 +929,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     // the global stores are whole 256-byte row segments.
     l += __shfl_xor(l, 32);
     const float rl = 1.0f / l;
+    if constexpr (DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // (a workgroup with an empty list never waited for its guessed tile)
     __syncthreads(); // every wave is done with the last K/V tile
     {
         float *so = reinterpret_cast<float *>(smem) + wave * 32 * LDO;
