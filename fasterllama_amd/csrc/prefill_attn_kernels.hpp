@@ -810,6 +810,13 @@ void prefill_attn_f16_kernel(const PrefillParams p)
             }
 
             if constexpr (DMA) {
+                // The compiler does not see the direct loads, so its wait for the mask entries counts them as
+                // landed ones: with the request for tile t+2 in flight behind the mask loads it would wait for
+                // that tile as well.  The mask entries are therefore waited for first (tile t+1, requested a
+                // tile ago, is all that is older).
+                if constexpr (HAS_MASK) {
+                    if (special) asm volatile("" : "+v"(st));
+                }
                 if (i + 2 < n) dma((int)(e2 >> 8), (buf + 2) % NBUF); // the buffer of tile t-1
             } else if (i + 1 < n) {
                 commit(buf ^ 1);
@@ -861,6 +868,21 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                         }
                     __builtin_amdgcn_sched_barrier(0);
                 }
+                // Without the full prefetch the V operands are read one output tile ahead of the products that
+                // use them, and the first set before the softmax: left to itself the compiler reads each pair
+                // right before its product, and every product waits out an LDS round trip.
+                half4 vst[2][4];
+                auto v_stage = [&](int stage, int dt) {
+#pragma unroll
+                    for (int u = 0; u < 2; ++u) {
+                        vst[stage][2 * u] = v_operand(buf, 16 * u, dt);
+                        vst[stage][2 * u + 1] = v_operand(buf, 16 * u + 8, dt);
+                    }
+                };
+                if constexpr (!PF_VA) {
+                    v_stage(0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
                 // Softmax update of this lane's query (decoder_kernels.cu:811-833 in base 2).  The reference
                 // maximum m may lag the true running maximum by up to kLazyMax (weights up to 2^kLazyMax,
                 // well inside fp16 and exact in the final ratio): with 32 queries per wave some maximum
@@ -891,16 +913,22 @@ void prefill_attn_f16_kernel(const PrefillParams p)
 
                 // O^T += V^T P^T, 16 keys per MFMA
 #pragma unroll
-                for (int dt = 0; dt < NDT; ++dt)
+                for (int dt = 0; dt < NDT; ++dt) {
+                    if constexpr (!PF_VA) {
+                        if (dt + 1 < NDT) v_stage((dt + 1) & 1, dt + 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
 #pragma unroll
                     for (int u = 0; u < 2; ++u) {
-                        const half4 lo = PF_VA ? vlo[PF_VA ? dt : 0][u] : v_operand(buf, 16 * u, dt);
-                        const half4 hi = PF_VA ? vhi[PF_VA ? dt : 0][u] : v_operand(buf, 16 * u + 8, dt);
+                        const half4 lo = PF_VA ? vlo[PF_VA ? dt : 0][u] : vst[dt & 1][2 * u];
+                        const half4 hi = PF_VA ? vhi[PF_VA ? dt : 0][u] : vst[dt & 1][2 * u + 1];
                         half8 va;
                         va[0] = lo[0]; va[1] = lo[1]; va[2] = lo[2]; va[3] = lo[3];
                         va[4] = hi[0]; va[5] = hi[1]; va[6] = hi[2]; va[7] = hi[3];
                         ot[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pr[u], ot[dt], 0, 0, 0);
                     }
+                    if constexpr (!PF_VA) __builtin_amdgcn_sched_barrier(0);
+                }
             }
 
             e0 = e1;
