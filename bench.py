@@ -432,6 +432,7 @@ def calibrate(args) -> int:
     lib.fl_calib_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     lib.fl_calib_mfma.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     lib.fl_calib_empty.argtypes = [C.c_void_p]
+    lib.fl_calib_coexec.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     dev = torch.device("cuda:0")
     stream = torch.cuda.current_stream(dev)
     sp = C.c_void_p(stream.cuda_stream)
@@ -481,6 +482,19 @@ def calibrate(args) -> int:
                                  "waves_per_simd": wgs_per_cu, "operands": "random in [-2,2]" if rnd else "zeros",
                                  "TFLOPs": round(flops / (ms * 1e-3) / 1e12, 1)})
         out.update(compute_units=cus, results=rows)
+    elif args.calib == "coexec":
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        iters = 20000
+        rows = []
+        for n_cu in (cus // 16, cus):
+            row = {"compute_units_busy": n_cu}
+            for what, name in ((1, "matrix_wave_alone"), (2, "vector_wave_alone"), (3, "both_on_one_simd")):
+                ms = timed(lambda: ok(lib.fl_calib_coexec(what, n_cu, iters, sink.data_ptr(), sp)), 3)
+                row[name + "_ns_per_block"] = round(ms * 1e6 / iters, 1)
+            rows.append(row)
+        out.update(block="matrix wave: 8 dependent v_mfma_f32_32x32x16_f16 (256 cycles); vector wave: 48 v_fma_f32 + "
+                         "16 v_exp_f32 on 16 independent values; one wave of each kind per SIMD, one workgroup per CU",
+                   results=rows)
     elif args.calib == "launch":
         ms = timed(lambda: ok(lib.fl_calib_empty(sp)), 2000)
         out.update(empty_kernel_us_per_launch=round(ms * 1e3, 3),
@@ -506,10 +520,11 @@ def main() -> int:
     ap.add_argument("--no-others", action="store_true",
                     help="skip the other_configs object (the remaining configurations, measured in the same run "
                          "with the headline workload)")
-    ap.add_argument("--calib", choices=["copy", "read", "mfma", "launch"],
+    ap.add_argument("--calib", choices=["copy", "read", "mfma", "coexec", "launch"],
                     help="measurement-only legs, then exit.  copy: a plain 1 GiB -> 1 GiB elementwise copy (for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings); read: 2 GiB streaming read, plain and non-temporal "
-                         "loads; mfma: register-only MFMA loops; launch: empty-kernel launch cadence")
+                         "loads; mfma: register-only MFMA loops; coexec: a matrix wave and a vector wave per SIMD, alone and together, "
+                         "on a sixteenth of the CUs and on all of them; launch: empty-kernel launch cadence")
     ap.add_argument("--calib-copy", action="store_true", help="same as --calib copy")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
     ap.add_argument("--prefill-mask", default="causal", choices=["causal", "causal-1e5", "block-causal", "none"],

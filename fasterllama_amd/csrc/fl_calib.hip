@@ -5,6 +5,9 @@
 //                          one workgroup per contiguous slice (the access pattern of the decode step)
 //   fl_calib_empty         a kernel that does nothing (launch cadence of back-to-back dependent launches)
 //   fl_calib_mfma_f16/f32  register-only loops of v_mfma_f32_32x32x16_f16 / v_mfma_f32_32x32x2_f32
+//   fl_calib_coexec        one wave of matrix work and one wave of vector (fma + exp2) work per SIMD, each alone
+//                          and both together, on a chosen number of CUs: how far the two pipes overlap, and
+//                          what chip-wide load does to the clock
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -95,6 +98,51 @@ __global__ __launch_bounds__(256) void mfma_f32_kernel(float *sink, int iters, i
     if (s == 123.456f) sink[0] = s;
 }
 
+// Workgroup of 8 waves, one workgroup per CU (the dynamic LDS size sees to that): waves 0-3 (one per SIMD) run
+// chains of 8 dependent v_mfma_f32_32x32x16_f16 (8 x 32 cycles), waves 4-7 blocks of 48 v_fma_f32 + 16 v_exp_f32
+// over 16 independent values (the instruction mix of a softmax update).  what: 1 matrix waves only, 2 vector
+// waves only, 3 both.
+__global__ __launch_bounds__(512) void coexec_kernel(float *sink, int iters, int what)
+{
+    extern __shared__ char one_workgroup_per_cu[];
+    const int wave = threadIdx.x >> 6;
+    float r = 0.f;
+    if (wave < 4) {
+        if (what & 1) {
+            half8 a, b;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                a[i] = (_Float16)lane_value(threadIdx.x * 16u + i, true);
+                b[i] = (_Float16)lane_value(threadIdx.x * 16u + 8u + i, true);
+            }
+            floatx16 c;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) c[v] = 0.f;
+            for (int it = 0; it < iters; ++it)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) c = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) r += c[v];
+        }
+    } else if (what & 2) {
+        float x[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) x[v] = lane_value(threadIdx.x * 16u + v, true);
+        const float s = 0.999f, m = 0.001f;
+        for (int it = 0; it < iters; ++it) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) x[v] = __builtin_amdgcn_exp2f(fmaf(x[v], s, m));
+#pragma unroll
+            for (int k = 0; k < 2; ++k)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) x[v] = fmaf(x[v], s, m);
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) r += x[v];
+    }
+    if (r == 123.456f) sink[0] = r;
+}
+
 } // namespace
 
 extern "C" {
@@ -127,6 +175,18 @@ int fl_calib_mfma(int fp32, int blocks, int iters, int random_operands, float *s
         hipLaunchKernelGGL(mfma_f32_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), sink, iters, random_operands);
     else
         hipLaunchKernelGGL(mfma_f16_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), sink, iters, random_operands);
+    return (int)hipGetLastError();
+}
+
+// cus workgroups (one per CU); every matrix wave issues 8 * iters MFMAs, every vector wave 64 * iters
+// vector instructions.  what: 1 matrix waves, 2 vector waves, 3 both.
+int fl_calib_coexec(int what, int cus, int iters, float *sink, void *stream)
+{
+    if (!sink || cus <= 0 || iters <= 0 || what < 1 || what > 3) return (int)hipErrorInvalidValue;
+    const int lds = 96 * 1024;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(coexec_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    hipLaunchKernelGGL(coexec_kernel, dim3(cus), dim3(512), lds, static_cast<hipStream_t>(stream), sink, iters, what);
     return (int)hipGetLastError();
 }
 

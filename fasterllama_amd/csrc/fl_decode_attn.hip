@@ -170,6 +170,9 @@ void make_plan(const fl_attn_desc *d, int ctx, bool ragged, fl_attn_plan *plan)
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// Row stride of the persistent mask tile class table: the 32-row blocks of one key tile, padded to whole words.
+size_t class_table_ld(int total_len) { return align_up(((size_t)total_len + 31) / 32, 4); }
+
 // Kernel launch that reports its own status: hipLaunchKernel returns the error of this launch,
 // whereas hipGetLastError would also return (and clear) an error left behind by an earlier,
 // unrelated HIP call of the calling thread.
@@ -625,8 +628,9 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     p.freq_cis = io->freq_cis; p.attn_mask = io->attn_mask;
     p.tile_class = reinterpret_cast<uint32_t *>(ws + wl.tile_class);
     if (io->mask_tile_classes && io->attn_mask && io->mask_ld >= L && io->start_pos % 32 == 0) {
+        if ((reinterpret_cast<uintptr_t>(io->mask_tile_classes) & 3u) != 0) return FL_ATTN_ERR_ALIGNMENT; // read a word at a time
         p.class_table = static_cast<const uint8_t *>(io->mask_tile_classes);
-        p.class_ld = (L + 31) / 32;
+        p.class_ld = (int32_t)class_table_ld(L);
     }
     p.out = io->out ? io->out : reinterpret_cast<float *>(ws + wl.tmp_out);
     p.inp_scale = io->qkv_inp_scale; p.wq_scale = io->q_weight_scale;
@@ -654,7 +658,7 @@ int fl_prefill_mask_classes_bytes(const fl_attn_desc *desc, size_t *bytes)
     int st = validate_desc(desc);
     if (st != FL_ATTN_OK) return st;
     const size_t n = ((size_t)desc->total_len + 31) / 32;
-    *bytes = n * n;
+    *bytes = n * class_table_ld(desc->total_len);
     return FL_ATTN_OK;
 }
 
@@ -667,10 +671,11 @@ int fl_prefill_mask_classify(const fl_attn_desc *desc, const float *attn_mask, i
     const int L = desc->total_len;
     const size_t n = ((size_t)L + 31) / 32;
     if (mask_ld < L) return FL_ATTN_ERR_ARGUMENT;
-    if (classes_bytes < n * n) return FL_ATTN_ERR_WORKSPACE;
+    if (classes_bytes < n * class_table_ld(L)) return FL_ATTN_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(classes) & 3u) != 0) return FL_ATTN_ERR_ALIGNMENT;
     if (n > 65535) return FL_ATTN_ERR_SHAPE;
     if (!check_hip(launch(flattn::mask_class_table_kernel, dim3((unsigned)n, (unsigned)n), dim3(64), static_cast<hipStream_t>(hip_stream),
-                          attn_mask, mask_ld, L, L, static_cast<uint8_t *>(classes), (int)n)))
+                          attn_mask, mask_ld, L, L, static_cast<uint8_t *>(classes), (int)class_table_ld(L))))
         return FL_ATTN_ERR_HIP;
     return FL_ATTN_OK;
 }

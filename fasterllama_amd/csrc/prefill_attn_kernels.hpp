@@ -126,16 +126,26 @@ constexpr uint32_t kTileSkip = 0, kTileZero = 1, kTileMixed = 2; // mask tile cl
 
 // Classes of key tile t for the four 32-query sub-blocks of 128-query block qb, one per byte: from the words
 // this call's classify kernel wrote, or from the caller's persistent table over the whole mask (one byte per
-// 32-row block x 32-key tile, rows in blocks of 32 from mask row 0; start_pos is a multiple of 32 then).
+// 32-key tile x 32-row block, rows in blocks of 32 from mask row 0; start_pos is a multiple of 32 then).  The
+// table keeps the row blocks of one key tile together (byte t * class_ld + row block, class_ld a multiple of 4),
+// so the four bytes are one aligned word whenever start_pos is a multiple of 128.
 __device__ __forceinline__ uint32_t tile_class_word(const PrefillParams &p, int qb, int t, int NT)
 {
     if (p.class_table) {
-        const uint8_t *row = p.class_table + (size_t)(p.start_pos / 32 + 4 * qb) * p.class_ld + t;
+        const int rb0 = p.start_pos / 32 + 4 * qb;
+        const uint8_t *e = p.class_table + (size_t)t * p.class_ld + rb0;
         uint32_t w = 0;
+        if ((rb0 & 3) == 0) {
+            w = *reinterpret_cast<const uint32_t *>(e);
+        } else {
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-            if (qb * kPrefillQueriesPerBlock + 32 * k < p.S) w |= (uint32_t)row[(size_t)k * p.class_ld] << (8 * k);
-        return w; // sub-blocks beyond the prompt: kTileSkip
+            for (int k = 0; k < 4; ++k)
+                if (rb0 + k < p.class_ld) w |= (uint32_t)e[k] << (8 * k);
+        }
+#pragma unroll
+        for (int k = 1; k < 4; ++k) // sub-blocks beyond the prompt (their table bytes may be padding): kTileSkip
+            if (qb * kPrefillQueriesPerBlock + 32 * k >= p.S) w &= ~(0xffu << (8 * k));
+        return w;
     }
     return p.tile_class[(size_t)qb * NT + t];
 }
@@ -376,8 +386,8 @@ __global__ __launch_bounds__(256) void prefill_mask_classify_kernel(const Prefil
 }
 
 // The same classes for a WHOLE mask [rows, cols] (row stride mask_ld), once per mask instead of once per call:
-// one byte per (32-row block, 32-key tile); entries past the last row / column repeat the last one.
-// grid = (ceil(cols/32), ceil(rows/32)), block = 64.
+// one byte per (32-key tile, 32-row block) at table[tile * table_ld + row block]; entries past the last row /
+// column repeat the last one.  grid = (ceil(cols/32), ceil(rows/32)), block = 64.
 __global__ __launch_bounds__(64) void mask_class_table_kernel(const float *mask, int64_t mask_ld, int rows, int cols,
                                                               uint8_t *table, int table_ld)
 {
@@ -393,7 +403,7 @@ __global__ __launch_bounds__(64) void mask_class_table_kernel(const float *mask,
         open |= !(v <= kMaskedBelow);       // a NaN entry keeps the tile
     }
     const uint32_t cls = __ballot(open) == 0ull ? kTileSkip : (__ballot(nonzero != 0u) == 0ull ? kTileZero : kTileMixed);
-    if (lane == 0) table[(size_t)rb * table_ld + t] = (uint8_t)cls;
+    if (lane == 0) table[(size_t)t * table_ld + rb] = (uint8_t)cls;
 }
 
 // ---------------------------------------------------------------- fp16 caches: fp16 MFMA
