@@ -658,64 +658,111 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         if (tid < first_c1) w_first = tile_class_word(p, qb, tid, NT);
     }
 
-    // Rotated queries of the workgroup: loaded and rotated cooperatively (16 lanes per 256-byte row, so
-    // the [B,S,H,D] rows are read whole), rounded once to fp16 as MFMA operands, and handed to their
-    // lanes through LDS.  Reading them per lane instead — 32 rows a wave, 16 bytes a lane — keeps the
-    // texture units busy for longer than ten key tiles take.
+    // Rotated queries.  Every wave loads and rotates ITS OWN 32 queries cooperatively (CPR lanes per row, so the
+    // [B,S,H,D] rows are read whole; reading them per lane instead — 32 rows a wave, 16 bytes a lane — keeps the
+    // texture units busy for longer than ten key tiles take), rounds them once to fp16 as MFMA operands and turns
+    // them into the operand layout through its own slice of LDS: no workgroup barrier on the way.
     half8 qreg[NC];
     half8 qlo[QSPLIT ? NC : 1]; // remainders q - fp16(q): the first product runs on the pair, see below
     {
         const int b = bh / p.H, h = bh % p.H;
         const int row0 = p.rope_row < 0 ? P : p.rope_row;
-        constexpr int QPT = kPrefillQueriesPerBlock * CPR / 256; // 16-byte chunks per thread
-        half8 lo_keep[QSPLIT ? QPT : 1];
-        // Every chunk is loaded unconditionally (rows past the prompt read the prompt's last row and are
-        // zeroed afterwards): with the loads under a branch the compiler waits for each chunk before it
-        // requests the next, eight memory round trips in a row (11 us per workgroup instead of 2.5).
-        float x[QPT][8];
-        auto load_queries = [&](auto i32_tag) { // one straight run of loads per input format
+        constexpr int QPL = 32 * CPR / 64;  // 16-byte chunks per lane
+        constexpr int RPI = 64 / CPR;       // query rows per load instruction
+        static_assert(64 % CPR == 0, "a lane keeps its column chunk over all its rows");
+        const int cc = lane % CPR, rl = lane / CPR;
+        const int q_first = qb * kPrefillQueriesPerBlock + wave * 32;
+        _Float16 *const sq = sQ + wave * 32 * LDQ;
+        float x[QPL][8];
+        // All loads of a batch are issued before the first value is used (rows past the prompt read the
+        // prompt's last row and are zeroed afterwards): left to the compiler, or with the loads under a branch,
+        // a wave waits for one chunk before it requests the next — up to eight memory round trips in a row.
+        auto load_queries = [&](auto i32_tag) {
+            constexpr bool I32 = decltype(i32_tag)::value != 0;
+            constexpr int BATCH = I32 && QPL > 1 ? QPL / 2 : QPL; // int32 accumulators: twice the registers
+            float4 w[2];
+            if constexpr (I32) {
+                w[0] = *reinterpret_cast<const float4 *>(p.wq_scale + h * D + cc * 8);
+                w[1] = *reinterpret_cast<const float4 *>(p.wq_scale + h * D + cc * 8 + 4);
+            }
 #pragma unroll
-            for (int j = 0; j < QPT; ++j) {
-                const int idx = tid + j * 256;
-                const int r = idx / CPR, cc = idx % CPR;
-                const int q = min(qb * kPrefillQueriesPerBlock + r, S - 1);
-                rotated_query_chunk<_Float16, 8, decltype(i32_tag)::value>(p, D, (int64_t)b * S + q, h, cc * 8, row0 + q, x[j]);
+            for (int j0 = 0; j0 < QPL; j0 += BATCH) {
+                half8 rh[I32 ? 1 : BATCH];
+                int4 ri[I32 ? BATCH : 1][2];
+                float sc[I32 ? BATCH : 1];
+                float4 rf[BATCH][2];
+#pragma unroll
+                for (int jj = 0; jj < BATCH; ++jj) {
+                    const int q = min(q_first + rl + (j0 + jj) * RPI, S - 1);
+                    const int64_t token = (int64_t)b * S + q;
+                    const size_t off = (size_t)(token * p.H + h) * D + cc * 8;
+                    if constexpr (I32) {
+                        const int4 *src = reinterpret_cast<const int4 *>(reinterpret_cast<const int32_t *>(p.q) + off);
+                        ri[jj][0] = src[0];
+                        ri[jj][1] = src[1];
+                        sc[jj] = p.inp_scale[token];
+                    } else {
+                        rh[jj] = *reinterpret_cast<const half8 *>(reinterpret_cast<const _Float16 *>(p.q) + off);
+                    }
+                    const float4 *fr = reinterpret_cast<const float4 *>(p.freq_cis + (size_t)(row0 + q) * D + cc * 8);
+                    rf[jj][0] = fr[0];
+                    rf[jj][1] = fr[1];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int jj = 0; jj < BATCH; ++jj) {
+                    float v[8];
+                    if constexpr (I32) { // decoder_kernels.cu:449-452
+                        const int a[8] = {ri[jj][0].x, ri[jj][0].y, ri[jj][0].z, ri[jj][0].w, ri[jj][1].x, ri[jj][1].y, ri[jj][1].z, ri[jj][1].w};
+                        const float ws[8] = {w[0].x, w[0].y, w[0].z, w[0].w, w[1].x, w[1].y, w[1].z, w[1].w};
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) v[i] = __fmul_rn(__fmul_rn((float)a[i], sc[jj]), ws[i]);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) v[i] = (float)rh[jj][i];
+                    }
+                    float *o = x[j0 + jj];
+                    rope_pair(v[0], v[1], rf[jj][0].x, rf[jj][0].y, o[0], o[1]);
+                    rope_pair(v[2], v[3], rf[jj][0].z, rf[jj][0].w, o[2], o[3]);
+                    rope_pair(v[4], v[5], rf[jj][1].x, rf[jj][1].y, o[4], o[5]);
+                    rope_pair(v[6], v[7], rf[jj][1].z, rf[jj][1].w, o[6], o[7]);
+                }
             }
         };
         if (p.inp_scale != nullptr) load_queries(std::integral_constant<int, 1>{});
         else load_queries(std::integral_constant<int, 0>{});
+        auto wave_sync = [] { // orders this wave's LDS writes and reads; the slice belongs to the wave alone
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        };
+        half8 lo_keep[QSPLIT ? QPL : 1];
 #pragma unroll
-        for (int j = 0; j < QPT; ++j) {
-            const int idx = tid + j * 256;
-            const int r = idx / CPR, cc = idx % CPR;
-            const bool valid = qb * kPrefillQueriesPerBlock + r < S;
+        for (int j = 0; j < QPL; ++j) {
+            const bool valid = q_first + rl + j * RPI < S;
             half8 hq;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 hq[i] = valid ? (_Float16)x[j][i] : (_Float16)0;
                 if constexpr (QSPLIT) lo_keep[j][i] = valid ? (_Float16)(x[j][i] - (float)hq[i]) : (_Float16)0;
             }
-            *reinterpret_cast<half8 *>(sQ + r * LDQ + cc * 8) = hq;
+            *reinterpret_cast<half8 *>(sq + (rl + j * RPI) * LDQ + cc * 8) = hq;
         }
-        __syncthreads();
+        wave_sync();
 #pragma unroll
-        for (int c = 0; c < NC; ++c)
-            qreg[c] = *reinterpret_cast<const half8 *>(sQ + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
-        __syncthreads();
+        for (int c = 0; c < NC; ++c) qreg[c] = *reinterpret_cast<const half8 *>(sq + qi * LDQ + 16 * c + 8 * hf);
         if constexpr (QSPLIT) {
+            wave_sync();
 #pragma unroll
-            for (int j = 0; j < QPT; ++j) {
-                const int idx = tid + j * 256;
-                *reinterpret_cast<half8 *>(sQ + (idx / CPR) * LDQ + (idx % CPR) * 8) = lo_keep[j];
-            }
-            __syncthreads();
+            for (int j = 0; j < QPL; ++j) *reinterpret_cast<half8 *>(sq + (rl + j * RPI) * LDQ + cc * 8) = lo_keep[j];
+            wave_sync();
 #pragma unroll
-            for (int c = 0; c < NC; ++c)
-                qlo[c] = *reinterpret_cast<const half8 *>(sQ + (wave * 32 + qi) * LDQ + 16 * c + 8 * hf);
-            __syncthreads();
+            for (int c = 0; c < NC; ++c) qlo[c] = *reinterpret_cast<const half8 *>(sq + qi * LDQ + 16 * c + 8 * hf);
         }
-        // the tile buffers behind the first are free for K and V
     }
+    // The slices lie in the tile buffers (behind the first one, on the direct path): every wave must be done with
+    // its own before a tile is stored there.  With a mask the barriers of the list build see to that.
+    if constexpr (!HAS_MASK) __syncthreads();
     int n_first = first_c1;
     if constexpr (HAS_MASK) n_first = build_list(0, first_c1, true, w_first);
     if (n_first > 0) {
