@@ -474,7 +474,9 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     // from LDS before the first product is issued (and, with the single fp16 query, the V operands before the
     // softmax), so LDS latency is paid once per tile and not once per pair of matrix instructions.  The
     // unmasked single-query instance is left alone: it fits 168 registers, runs THREE waves per SIMD and
-    // loses more from a fourth dozen of registers than it gains (B=8, S=1024: 0.221 ms against 0.240).
+    // loses more from a fourth dozen of registers than it gains (B=8, S=1024: 0.221 ms against 0.240).  The
+    // masked single-query instance is the other way round: squeezed into 168 registers without the prefetch
+    // it runs three waves per SIMD and is 5-10 % slower than with the prefetch at two.
     constexpr bool PF_KA = HAS_MASK || QSPLIT;
     constexpr bool PF_VA = HAS_MASK && !QSPLIT;
     constexpr int BN = kPrefillKeysPerStep; // 32
@@ -596,7 +598,8 @@ void prefill_attn_f16_kernel(const PrefillParams p)
 
     // Direct path.  One instruction moves 1 KB, four rows: lane -> row lane/16, 16-byte position lane%16.  Wave w
     // issues the blocks 2w and 2w+1 of K and of V.  The range check of the descriptor (rows at or beyond the
-    // context arrive as zeros) applies to the lane offset only, so the tile's slab is added to it.
+    // context arrive as zeros: a lane out of range writes 16 zero bytes into LDS, it does not skip its write)
+    // applies to the lane offset only, so the tile's slab is added to it.
     uint32_t dk_off[DMA ? 2 : 1], dv_off[DMA ? 2 : 1];
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     if constexpr (DMA) {

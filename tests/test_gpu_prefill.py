@@ -233,12 +233,13 @@ def test_prefill_dense_random_mask_f16(gpu):
     assert_out_close(out.cpu().numpy(), want, "f16", "dense random mask")
 
 
-def test_prefill_context_longer_than_one_tile_list_f16(gpu):
-    """More key tiles than one pass of the kernel's tile list holds (1024 tiles = 32768 keys).  The mask is a
-    single row shared by all queries (row stride 0): a key-padding mask that hides two long runs of keys."""
+@pytest.mark.parametrize("D", [32, 128])
+def test_prefill_context_longer_than_one_tile_list_f16(gpu, D):
+    """More key tiles than one pass of the kernel's tile list holds (1024 tiles = 32768 keys).  The
+    mask is a single row shared by all queries (row stride 0): a key-padding mask that hides two long runs of keys."""
     import torch
     from fasterllama_amd.decode_attn import PrefillAttention
-    B, H, D, L, S = 1, 1, 32, 33100, 96
+    B, H, L, S = 1, 1, 33100, 96
     P = L - S
     row = np.zeros(L, np.float32)
     row[64:20000] = -FMAX
