@@ -171,6 +171,65 @@ __device__ __forceinline__ void prefill_block_to_tile(int block, int BH, int QB,
     }
 }
 
+// The tiles of [c0, c1) that some wave of the workgroup (256 threads, 128 queries: block qb) needs, in order, as a
+// list in LDS: entry = tile << 8 | the four waves' classes (2 bits each).  Returns their number; ends with a
+// barrier.  w_first: this thread's class word of tile c0 + tid where the caller has loaded it already.
+__device__ __forceinline__ int build_tile_list(const PrefillParams &p, int qb, int c0, int c1, int NT, bool have_first,
+                                               uint32_t w_first, uint32_t *s_list, int *s_wave_cnt)
+{
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int count = 0;
+    for (int base = c0; base < c1; base += 256) {
+        const int t = base + tid;
+        uint32_t w = 0;
+        if (have_first && base == c0) w = w_first;
+        else if (t < c1) w = tile_class_word(p, qb, t, NT);
+        const bool active = w != 0u;
+        const unsigned long long bal = __ballot(active);
+        if (lane == 0) s_wave_cnt[wave] = __popcll(bal);
+        __syncthreads();
+        int off = count;
+        for (int k = 0; k < wave; ++k) off += s_wave_cnt[k];
+        if (active) {
+            const uint32_t packed = (w & 3u) | ((w >> 8) & 3u) << 2 | ((w >> 16) & 3u) << 4 | ((w >> 24) & 3u) << 6;
+            s_list[off + __popcll(bal & ((1ull << lane) - 1ull))] = (uint32_t)t << 8 | packed;
+        }
+        count += s_wave_cnt[0] + s_wave_cnt[1] + s_wave_cnt[2] + s_wave_cnt[3];
+        __syncthreads();
+    }
+    return count;
+}
+constexpr int kTileListCap = 1024; // tiles per pass over the context (32768 keys); longer contexts take several passes
+
+typedef int int4v __attribute__((ext_vector_type(4)));
+
+// Raw buffer descriptor over `bytes` bytes at base: loads at or beyond the end return zeros.
+__device__ __forceinline__ int4v raw_descriptor(const void *base, uint32_t bytes)
+{
+    const uint64_t a = reinterpret_cast<uint64_t>(base);
+    return int4v{(int)(uint32_t)a, (int)(uint32_t)(a >> 32), (int)bytes, 0x00020000};
+}
+
+// Two direct loads global -> LDS (buffer_load_dwordx4 ... lds: lane i's 16 bytes land at lds + 16 i; a lane whose
+// offset is out of the descriptor's range writes zeros).  Written as assembly on purpose: the compiler treats a
+// direct load as a store to LDS that any later LDS read may alias, and as pending work every workgroup barrier
+// must drain — it would put `s_waitcnt vmcnt(0)` before such reads and before each barrier, which waits for the
+// tile that was requested a moment ago and serialises the pipeline.  The callers wait (s_waitcnt vmcnt(n)) for
+// exactly the tile they are about to read.  M0 carries the LDS address; one wait state separates its write from
+// the load that uses it; it is the compiler's register elsewhere and is handed back as it was.
+__device__ __forceinline__ void direct_load_pair(uint32_t lds_a, uint32_t off_a, const int4v &desc_a, uint32_t lds_b,
+                                                 uint32_t off_b, const int4v &desc_b)
+{
+    uint32_t m0_saved;
+    asm volatile("s_mov_b32 %0, m0\n\t"
+                 "s_mov_b32 m0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, 0 offen lds\n\t"
+                 "s_mov_b32 m0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %5, %6, 0 offen lds\n\t"
+                 "s_mov_b32 m0, %0"
+                 : "=&s"(m0_saved)
+                 : "s"(lds_a), "v"(off_a), "s"(desc_a), "s"(lds_b), "v"(off_b), "s"(desc_b)
+                 : "memory");
+}
+
 // MFMA operand layouts used below (v_mfma_f32_32x32x2_f32, D += A(32x2) * B(2x32)):
 //   A: lane holds A[row = lane % 32][k = lane / 32];  B: lane holds B[k = lane / 32][col = lane % 32];
 //   D: register v of a lane holds D[row = 8*(v/4) + 4*(lane/32) + (v%4)][col = lane % 32].
@@ -186,14 +245,32 @@ void prefill_attn_kernel(const PrefillParams p)
     typedef typename Vec16<T>::type V;
     constexpr int VEC = Vec16<T>::N;
     constexpr int BN = kPrefillKeysPerStep;
-    constexpr int LDK = D + 4; // padded LDS row (floats): rows start 4 banks apart
     constexpr int NC = D / 8;
     constexpr int NDT = D / 32;
     constexpr int CPR = D / VEC; // 16-byte chunks per cache row
     static_assert(D % 32 == 0, "head size must be a multiple of 32");
+    static_assert(std::is_same<T, float>::value, "the FP32-MFMA kernel works on FP32 caches");
 
-    __shared__ float sK[BN][LDK];
-    __shared__ float sV[BN][LDK];
+    // D >= 64: the key tiles go from global memory straight into LDS, two buffers deep, so the next tile
+    // travels while this one is multiplied (128 MFMAs of 64 cycles per wave and tile: the products cover
+    // the memory latency with room to spare, and no register is spent on staging).  A direct load lays the
+    // lanes' 16-byte chunks down back to back — one instruction is 1 KB: RPI whole rows — so rows cannot
+    // be padded against bank conflicts; they are swizzled instead: K keeps chunk c of row r at c ^ (r & 15)
+    // (the 16 lanes of a 128-bit read pass, keys r..r+15 at one d, hit 16 different bank groups), V keeps it at
+    // c ^ 8 for the rows with bit 2 set (the two key rows of a 32-bit read, four apart, use different halves
+    // of the banks).  Each lane applies the swizzle to the GLOBAL address it loads from.
+    constexpr bool DMA = D >= 64;
+    constexpr int ROWB = D * 4;          // bytes per cache row
+    constexpr int RPI = 1024 / ROWB;     // rows per direct load
+    constexpr int NI = DMA ? BN / RPI / 4 : 1; // direct loads per wave, tile and matrix
+    constexpr uint32_t TILEB = BN * ROWB; // bytes of one K (or V) tile
+    constexpr int LDK = D + 4;           // staged path: padded LDS row (floats), rows start 4 banks apart
+    constexpr int SMEM_FLOATS = DMA ? 4 * BN * D : 2 * BN * LDK;
+    __shared__ __attribute__((aligned(16))) float smem[SMEM_FLOATS];
+    float (*sK)[LDK] = reinterpret_cast<float (*)[LDK]>(smem);            // staged path only
+    float (*sV)[LDK] = reinterpret_cast<float (*)[LDK]>(smem + BN * LDK); // staged path only
+    __shared__ uint32_t s_list[HAS_MASK && DMA ? kTileListCap : 1];
+    __shared__ int s_wave_cnt[4];
 
     const int BH = p.B * p.H;
     int qb, bh;
@@ -204,10 +281,41 @@ void prefill_attn_kernel(const PrefillParams p)
     const int qi = lane & 31, hf = lane >> 5;
     const int q_row = qb * kPrefillQueriesPerBlock + wave * 32 + qi;
     const bool q_ok = q_row < S;
+    const int NTC = (ctx + BN - 1) / BN;
+    const T *Kb = reinterpret_cast<const T *>(p.k_cache) + (size_t)bh * L * D;
+    const T *Vb = reinterpret_cast<const T *>(p.v_cache) + (size_t)bh * L * D;
+
+    // direct path: requests of one tile (tile t -> buffer buf); rows at or beyond the context arrive as zeros
+    const int4v Kdesc = raw_descriptor(Kb, (uint32_t)ctx * (uint32_t)ROWB), Vdesc = raw_descriptor(Vb, (uint32_t)ctx * (uint32_t)ROWB);
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    typedef __attribute__((address_space(3))) float *lds_float_ptr;
+    const uint32_t lds_wave = (uint32_t)(uintptr_t)(lds_float_ptr)smem + (uint32_t)(wave_u * NI) * 1024u;
+    uint32_t dk_off0 = 0, dv_off0 = 0;
+    if constexpr (DMA) {
+        const int r0 = wave * NI * RPI + lane / (64 / RPI), pc = lane % (64 / RPI);
+        dk_off0 = (uint32_t)(r0 * ROWB + ((pc ^ (r0 & 15)) << 4));
+        dv_off0 = (uint32_t)(r0 * ROWB + (pc << 4)); // bit 2 of the row comes from the load's index below
+    }
+    auto dma = [&](int t, int buf) {
+        const uint32_t slab = (uint32_t)t * TILEB; // part of the lane offset: the range check does not see a scalar offset
+#pragma unroll
+        for (int j = 0; j < NI; ++j) { // rows r0 + j * RPI: the swizzle terms of j touch bits of their own
+            const uint32_t k_off = (dk_off0 ^ (uint32_t)(((j * RPI) & 15) << 4)) + (uint32_t)(j * 1024) + slab;
+            const uint32_t v_off = (dv_off0 ^ (uint32_t)((((j * RPI) >> 2) & 1) << 7)) + (uint32_t)(j * 1024) + slab;
+            const uint32_t k_lds = lds_wave + (uint32_t)buf * 2u * TILEB + (uint32_t)(j * 1024);
+            direct_load_pair(k_lds, k_off, Kdesc, k_lds + TILEB, v_off, Vdesc);
+        }
+    };
+    // The tile list of the first pass and its first tile are requested before the queries.
+    const int first_c1 = min(kTileListCap, NTC);
+    int n_first = first_c1;
+    if constexpr (DMA) {
+        if constexpr (HAS_MASK) n_first = build_tile_list(p, qb, 0, first_c1, NTC, false, 0u, s_list, s_wave_cnt);
+        if (n_first > 0) dma(HAS_MASK ? (int)(__builtin_amdgcn_readfirstlane(s_list[0]) >> 8) : 0, 0);
+    }
 
     float qreg[NC][4];
     {
-        static_assert(std::is_same<T, float>::value, "the FP32-MFMA kernel works on FP32 caches");
         const int64_t token = (int64_t)(bh / p.H) * S + (q_ok ? q_row : 0);
         const int row = (p.rope_row < 0 ? P : p.rope_row) + (q_ok ? q_row : 0);
 #pragma unroll
@@ -224,64 +332,27 @@ void prefill_attn_kernel(const PrefillParams p)
         for (int v = 0; v < 16; ++v) ot[dt][v] = 0.f;
     float m = kMaxFloor, l = 0.f;
     const float *mrow = HAS_MASK ? p.attn_mask + (size_t)(P + (q_ok ? q_row : 0)) * p.mask_ld : nullptr;
-    const T *Kb = reinterpret_cast<const T *>(p.k_cache) + (size_t)bh * L * D;
-    const T *Vb = reinterpret_cast<const T *>(p.v_cache) + (size_t)bh * L * D;
     const float scale = p.scale;
 
-    // Mask tile classes (see prefill_mask_classify_kernel): a tile no wave of the workgroup needs is
-    // neither loaded nor multiplied, a wave skips the tiles it alone does not need, and the mask is
-    // only read where it is not all zero.  Each of these leaves every bit of the result as it is:
-    // the dropped terms are exp(v - max) == 0 and fma(s, scale, 0) == s*scale.
-    const int NTC = (ctx + BN - 1) / BN;
-    uint32_t word_next = HAS_MASK ? tile_class_word(p, qb, 0, NTC) : 0u;
+    // LDS addresses of the operands on the direct path (bytes from the tile buffer's start): the K operand of chunk
+    // c is one XOR away from k_swz; the V operand of output tile dt sits in the half of its 256 bytes that dt ^ hf names.
+    const uint32_t k_swz = (uint32_t)(qi * ROWB + ((hf ^ (qi & 15)) << 4));
+    const uint32_t v_lane = (uint32_t)(4 * hf * ROWB + qi * 4);
 
-    for (int k0 = 0; k0 < ctx; k0 += BN) {
-        uint32_t tc = kTileZero;
-        if constexpr (HAS_MASK) {
-            const uint32_t word = __builtin_amdgcn_readfirstlane(word_next);
-            if (k0 + BN < ctx) word_next = tile_class_word(p, qb, k0 / BN + 1, NTC); // in flight during this tile
-            if (word == 0u) continue;
-            tc = (word >> (8 * wave)) & 0xffu;
-        }
-        __syncthreads(); // every wave is done with the previous tile
-        for (int idx = tid; idx < BN * CPR; idx += 256) {
-            const int r = idx / CPR, cc = idx % CPR;
-            const int key = k0 + r;
-            float kf[VEC], vf[VEC];
-            if (key < ctx) {
-                const V kx = *reinterpret_cast<const V *>(Kb + (size_t)key * D + cc * VEC);
-                const V vx = *reinterpret_cast<const V *>(Vb + (size_t)key * D + cc * VEC);
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) { kf[i] = (float)kx[i]; vf[i] = (float)vx[i]; }
-            } else { // past the context: zeros, and the scores are forced to -inf below
-#pragma unroll
-                for (int i = 0; i < VEC; ++i) { kf[i] = 0.f; vf[i] = 0.f; }
-            }
-#pragma unroll
-            for (int i = 0; i < VEC; i += 4) {
-                *reinterpret_cast<float4 *>(&sK[r][cc * VEC + i]) = make_float4(kf[i], kf[i + 1], kf[i + 2], kf[i + 3]);
-                *reinterpret_cast<float4 *>(&sV[r][cc * VEC + i]) = make_float4(vf[i], vf[i + 1], vf[i + 2], vf[i + 3]);
-            }
-        }
-        // mask values of this lane's query, gathered straight from global memory: the FP32-MFMA kernel
-        // is matrix-core bound with every register in use, so the gather hides behind the products
-        // (staging the tile in LDS, as the fp16 kernel does, costs occupancy here: 1.53 -> 2.09 ms)
-        float mk[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int key = k0 + 8 * (v / 4) + 4 * hf + (v % 4);
-            mk[v] = (HAS_MASK && tc == kTileMixed && key < ctx) ? mrow[key] : 0.f;
-        }
-        __syncthreads();
-        if (tc == kTileSkip) continue; // wave-uniform; the barriers above are this iteration's only ones
-
+    // One key tile (keys k0..k0+31, class tc for this wave) against the wave's 32 queries; the tile's K rows at
+    // kt, V rows at vt (staged path: padded rows; direct path: swizzled rows in buffer `buf`).
+    auto multiply_tile = [&](int k0, uint32_t tc, const float (&mk)[16], auto direct_tag, int buf) {
+        constexpr bool DIRECT = decltype(direct_tag)::value;
+        const char *kt = reinterpret_cast<const char *>(smem) + (DIRECT ? (uint32_t)buf * 2u * TILEB : 0u);
+        const char *vt = kt + TILEB;
         // S^T tile: 32 keys x 32 queries, contraction over D
         floatx16 st;
 #pragma unroll
         for (int v = 0; v < 16; ++v) st[v] = 0.f;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
-            const float4 ka = *reinterpret_cast<const float4 *>(&sK[qi][8 * c + 4 * hf]);
+            const float4 ka = DIRECT ? *reinterpret_cast<const float4 *>(kt + (k_swz ^ (uint32_t)(c << 5)))
+                                     : *reinterpret_cast<const float4 *>(&sK[qi][8 * c + 4 * hf]);
             st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.x, qreg[c][0], st, 0, 0, 0);
             st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.y, qreg[c][1], st, 0, 0, 0);
             st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.z, qreg[c][2], st, 0, 0, 0);
@@ -319,9 +390,100 @@ void prefill_attn_kernel(const PrefillParams p)
         for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
             for (int t = 0; t < 16; ++t) {
-                const float va = sV[8 * (t / 4) + 4 * hf + (t % 4)][32 * dt + qi];
+                const float va = DIRECT ? *reinterpret_cast<const float *>(vt + v_lane + (uint32_t)((((dt & 1) ^ hf) << 7) + (dt >> 1) * 256 +
+                                                                                                   (8 * (t / 4) + (t % 4)) * ROWB))
+                                        : sV[8 * (t / 4) + 4 * hf + (t % 4)][32 * dt + qi];
                 ot[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(va, sc[t], ot[dt], 0, 0, 0);
             }
+        (void)tc;
+    };
+    // mask values of this lane's query, gathered straight from global memory: the FP32-MFMA kernel
+    // is matrix-core bound with every register in use, so the gather hides behind the products
+    // (staging the tile in LDS, as the fp16 kernel does, costs occupancy here: 1.53 -> 2.09 ms)
+    auto gather_mask = [&](int k0, uint32_t tc, float (&mk)[16]) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int key = k0 + 8 * (v / 4) + 4 * hf + (v % 4);
+            mk[v] = (HAS_MASK && tc == kTileMixed && key < ctx) ? mrow[key] : 0.f;
+        }
+    };
+
+    // Mask tile classes (see prefill_mask_classify_kernel): a tile no wave of the workgroup needs is
+    // neither loaded nor multiplied, a wave skips the tiles it alone does not need, and the mask is
+    // only read where it is not all zero.  Each of these leaves every bit of the result as it is:
+    // the dropped terms are exp(v - max) == 0 and fma(s, scale, 0) == s*scale.
+    if constexpr (DMA) {
+        auto list_entry = [&](int c0, int i) -> uint32_t { // without a mask every tile is needed and every class is ZERO
+            if constexpr (HAS_MASK) return s_list[i];
+            else return (uint32_t)(c0 + i) << 8 | 0x55u;
+        };
+        for (int c0 = 0; c0 < NTC; c0 += kTileListCap) {
+            const int c1 = min(c0 + kTileListCap, NTC);
+            int n = c1 - c0;
+            if (c0 == 0) n = n_first; // built, and its first tile requested, above
+            else if constexpr (HAS_MASK) n = build_tile_list(p, qb, c0, c1, NTC, false, 0u, s_list, s_wave_cnt); // ends with a barrier
+            else __syncthreads();                                                                              // both buffers are free
+            if (n == 0) continue;
+            uint32_t e0 = __builtin_amdgcn_readfirstlane(list_entry(c0, 0));
+            uint32_t e1 = n > 1 ? __builtin_amdgcn_readfirstlane(list_entry(c0, 1)) : 0u;
+            uint32_t e2 = n > 2 ? list_entry(c0, 2) : 0u;
+            if (c0 > 0) dma((int)(e0 >> 8), 0);
+            auto tile_step = [&](int i, auto buf_tag) {
+                constexpr int buf = decltype(buf_tag)::value;
+                const int k0 = (int)(e0 >> 8) * BN;
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's part of the tile has landed
+                __syncthreads();                                  // all of it is visible; every wave is done with the other buffer
+                uint32_t tc = kTileZero;
+                if constexpr (HAS_MASK) tc = __builtin_amdgcn_readfirstlane((e0 >> (2 * wave)) & 3u);
+                float mk[16];
+                gather_mask(k0, tc, mk);
+                if (i + 1 < n) dma((int)(e1 >> 8), buf ^ 1);
+                if (tc != kTileSkip) multiply_tile(k0, tc, mk, std::integral_constant<bool, true>{}, buf);
+                e0 = e1;
+                e1 = __builtin_amdgcn_readfirstlane(e2);
+                e2 = i + 3 < n ? list_entry(c0, i + 3) : 0u;
+            };
+            for (int i = 0; i < n; i += 2) {
+                tile_step(i, std::integral_constant<int, 0>{});
+                if (i + 1 < n) tile_step(i + 1, std::integral_constant<int, 1>{});
+            }
+        }
+    } else {
+        uint32_t word_next = HAS_MASK ? tile_class_word(p, qb, 0, NTC) : 0u;
+        for (int k0 = 0; k0 < ctx; k0 += BN) {
+            uint32_t tc = kTileZero;
+            if constexpr (HAS_MASK) {
+                const uint32_t word = __builtin_amdgcn_readfirstlane(word_next);
+                if (k0 + BN < ctx) word_next = tile_class_word(p, qb, k0 / BN + 1, NTC); // in flight during this tile
+                if (word == 0u) continue;
+                tc = (word >> (8 * wave)) & 0xffu;
+            }
+            __syncthreads(); // every wave is done with the previous tile
+            for (int idx = tid; idx < BN * CPR; idx += 256) {
+                const int r = idx / CPR, cc = idx % CPR;
+                const int key = k0 + r;
+                float kf[VEC], vf[VEC];
+                if (key < ctx) {
+                    const V kx = *reinterpret_cast<const V *>(Kb + (size_t)key * D + cc * VEC);
+                    const V vx = *reinterpret_cast<const V *>(Vb + (size_t)key * D + cc * VEC);
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) { kf[i] = (float)kx[i]; vf[i] = (float)vx[i]; }
+                } else { // past the context: zeros, and the scores are forced to -inf below
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) { kf[i] = 0.f; vf[i] = 0.f; }
+                }
+#pragma unroll
+                for (int i = 0; i < VEC; i += 4) {
+                    *reinterpret_cast<float4 *>(&sK[r][cc * VEC + i]) = make_float4(kf[i], kf[i + 1], kf[i + 2], kf[i + 3]);
+                    *reinterpret_cast<float4 *>(&sV[r][cc * VEC + i]) = make_float4(vf[i], vf[i + 1], vf[i + 2], vf[i + 3]);
+                }
+            }
+            float mk[16];
+            gather_mask(k0, tc, mk);
+            __syncthreads();
+            if (tc == kTileSkip) continue; // wave-uniform; the barriers above are this iteration's only ones
+            multiply_tile(k0, tc, mk, std::integral_constant<bool, false>{}, 0);
+        }
     }
 
     l += __shfl_xor(l, 32);
@@ -464,7 +626,6 @@ __device__ __forceinline__ float max16(const floatx16 &a)
 //
 // With a mask, tiles are processed according to their class (see above): each workgroup compacts the
 // tiles some wave of it needs into a list in LDS, and tiles that every wave skips are not even loaded.
-constexpr int kTileListCap = 1024; // tiles per pass over the context (32768 keys); longer contexts take several passes
 
 template <int D, bool HAS_MASK, bool QSPLIT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8)))
@@ -525,31 +686,10 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     const int qi = lane & 31, hf = lane >> 5;
     const int q_row = qb * kPrefillQueriesPerBlock + wave * 32 + qi;
 
-    // The tiles of [c0, c1) that some wave of this workgroup needs, in order, as a list in LDS:
-    // entry = tile << 8 | the four waves' classes (2 bits each).  Built once per chunk of
+    // The tiles some wave of this workgroup needs, as a list in LDS (build_tile_list): built once per pass of
     // kTileListCap tiles, so the loop below never chases a class word through memory.
-    // (w_first: this thread's class word of tile c0 + tid where the caller has loaded it already)
     auto build_list = [&](int c0, int c1, bool have_first, uint32_t w_first) -> int {
-        int count = 0;
-        for (int base = c0; base < c1; base += 256) {
-            const int t = base + tid;
-            uint32_t w = 0;
-            if (have_first && base == c0) w = w_first;
-            else if (t < c1) w = tile_class_word(p, qb, t, NT);
-            const bool active = w != 0u;
-            const unsigned long long bal = __ballot(active);
-            if (lane == 0) s_wave_cnt[wave] = __popcll(bal);
-            __syncthreads();
-            int off = count;
-            for (int k = 0; k < wave; ++k) off += s_wave_cnt[k];
-            if (active) {
-                const uint32_t packed = (w & 3u) | ((w >> 8) & 3u) << 2 | ((w >> 16) & 3u) << 4 | ((w >> 24) & 3u) << 6;
-                s_list[off + __popcll(bal & ((1ull << lane) - 1ull))] = (uint32_t)t << 8 | packed;
-            }
-            count += s_wave_cnt[0] + s_wave_cnt[1] + s_wave_cnt[2] + s_wave_cnt[3];
-            __syncthreads();
-        }
-        return count;
+        return build_tile_list(p, qb, c0, c1, NT, have_first, w_first, s_list, s_wave_cnt);
     };
     // entry i of the current chunk; without a mask every tile is needed and every class is ZERO
     auto list_entry = [&](int c0, int i) -> uint32_t {
@@ -610,18 +750,10 @@ void prefill_attn_f16_kernel(const PrefillParams p)
             dv_off[j] = (uint32_t)(r * 256 + ((((pc >> 2) ^ (r & 3)) << 2 | (pc & 3)) << 4));
         }
     }
-    // The loads are written as assembly on purpose.  The compiler treats a direct load as a store to LDS that
-    // any later LDS read may alias, and as pending work every workgroup barrier must drain: it would put
-    // `s_waitcnt vmcnt(0)` before the transposing reads and before each barrier, which waits for the tile that
-    // was requested a moment ago and serialises the pipeline.  The loop below waits for exactly the tile it is
-    // about to read (s_waitcnt vmcnt(4): the newer tile's four loads may stay in flight) before its barrier.
-    // M0 carries the LDS address of the block; one wait state separates its write from the load that uses it.
-    typedef int int4v __attribute__((ext_vector_type(4)));
-    auto raw_descriptor = [&](const _Float16 *base) -> int4v {
-        const uint64_t a = reinterpret_cast<uint64_t>(base);
-        return int4v{(int)(uint32_t)a, (int)(uint32_t)(a >> 32), (int)((uint32_t)ctx * (uint32_t)(D * 2)), 0x00020000};
-    };
-    const int4v Kdesc = raw_descriptor(Kb), Vdesc = raw_descriptor(Vb);
+    // (direct_load_pair: assembly, because the compiler would wait for every direct load in flight before each LDS
+    // read that might alias it and before each barrier.)  The loop below waits for exactly the tile it is about to
+    // read (s_waitcnt vmcnt(4): the newer tile's four loads may stay in flight) before its barrier.
+    const int4v Kdesc = raw_descriptor(Kb, (uint32_t)ctx * (uint32_t)(D * 2)), Vdesc = raw_descriptor(Vb, (uint32_t)ctx * (uint32_t)(D * 2));
     typedef __attribute__((address_space(3))) _Float16 *lds_half_ptr;
     const uint32_t lds_tiles = (uint32_t)(uintptr_t)(lds_half_ptr)smem + (uint32_t)wave_u * 2048u; // this wave's blocks
     auto dma = [&](int t, int buf) {
@@ -629,15 +761,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const uint32_t k_lds = lds_tiles + (uint32_t)buf * kTileBytes + (uint32_t)(j * 1024);
-            const uint32_t v_lds = k_lds + kVOff;
-            uint32_t m0_saved; // M0 is the compiler's to use elsewhere: hand it back as it was
-            asm volatile("s_mov_b32 %0, m0\n\t"
-                         "s_mov_b32 m0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, 0 offen lds\n\t"
-                         "s_mov_b32 m0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %5, %6, 0 offen lds\n\t"
-                         "s_mov_b32 m0, %0"
-                         : "=&s"(m0_saved)
-                         : "s"(k_lds), "v"(dk_off[DMA ? j : 0] + slab), "s"(Kdesc), "s"(v_lds), "v"(dv_off[DMA ? j : 0] + slab), "s"(Vdesc)
-                         : "memory");
+            direct_load_pair(k_lds, dk_off[DMA ? j : 0] + slab, Kdesc, k_lds + kVOff, dv_off[DMA ? j : 0] + slab, Vdesc);
         }
     };
     // LDS addresses of the operands.  Padded layout: plain rows.  Swizzled layout: K chunk 2c+hf of row qi sits
