@@ -296,7 +296,7 @@ void prefill_attn_kernel(const PrefillParams p)
         dk_off0 = (uint32_t)(r0 * ROWB + ((pc ^ (r0 & 15)) << 4));
         dv_off0 = (uint32_t)(r0 * ROWB + (pc << 4)); // bit 2 of the row comes from the load's index below
     }
-    auto dma = [&](int t, int buf) {
+    auto dma = [&](int t, int buf) __attribute__((always_inline)) {
         const uint32_t slab = (uint32_t)t * TILEB; // part of the lane offset: the range check does not see a scalar offset
 #pragma unroll
         for (int j = 0; j < NI; ++j) { // rows r0 + j * RPI: the swizzle terms of j touch bits of their own
@@ -341,7 +341,7 @@ void prefill_attn_kernel(const PrefillParams p)
 
     // One key tile (keys k0..k0+31, class tc for this wave) against the wave's 32 queries; the tile's K rows at
     // kt, V rows at vt (staged path: padded rows; direct path: swizzled rows in buffer `buf`).
-    auto multiply_tile = [&](int k0, uint32_t tc, const float (&mk)[16], auto direct_tag, int buf) {
+    auto multiply_tile = [&](int k0, uint32_t tc, const float (&mk)[16], auto direct_tag, int buf) __attribute__((always_inline)) {
         constexpr bool DIRECT = decltype(direct_tag)::value;
         const char *kt = reinterpret_cast<const char *>(smem) + (DIRECT ? (uint32_t)buf * 2u * TILEB : 0u);
         const char *vt = kt + TILEB;
@@ -400,7 +400,7 @@ void prefill_attn_kernel(const PrefillParams p)
     // mask values of this lane's query, gathered straight from global memory: the FP32-MFMA kernel
     // is matrix-core bound with every register in use, so the gather hides behind the products
     // (staging the tile in LDS, as the fp16 kernel does, costs occupancy here: 1.53 -> 2.09 ms)
-    auto gather_mask = [&](int k0, uint32_t tc, float (&mk)[16]) {
+    auto gather_mask = [&](int k0, uint32_t tc, float (&mk)[16]) __attribute__((always_inline)) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int key = k0 + 8 * (v / 4) + 4 * hf + (v % 4);
@@ -413,7 +413,7 @@ void prefill_attn_kernel(const PrefillParams p)
     // only read where it is not all zero.  Each of these leaves every bit of the result as it is:
     // the dropped terms are exp(v - max) == 0 and fma(s, scale, 0) == s*scale.
     if constexpr (DMA) {
-        auto list_entry = [&](int c0, int i) -> uint32_t { // without a mask every tile is needed and every class is ZERO
+        auto list_entry = [&](int c0, int i) __attribute__((always_inline)) -> uint32_t { // without a mask every tile is needed and every class is ZERO
             if constexpr (HAS_MASK) return s_list[i];
             else return (uint32_t)(c0 + i) << 8 | 0x55u;
         };
@@ -428,7 +428,7 @@ void prefill_attn_kernel(const PrefillParams p)
             uint32_t e1 = n > 1 ? __builtin_amdgcn_readfirstlane(list_entry(c0, 1)) : 0u;
             uint32_t e2 = n > 2 ? list_entry(c0, 2) : 0u;
             if (c0 > 0) dma((int)(e0 >> 8), 0);
-            auto tile_step = [&](int i, auto buf_tag) {
+            auto tile_step = [&](int i, auto buf_tag) __attribute__((always_inline)) {
                 constexpr int buf = decltype(buf_tag)::value;
                 const int k0 = (int)(e0 >> 8) * BN;
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wave's part of the tile has landed
@@ -688,11 +688,11 @@ void prefill_attn_f16_kernel(const PrefillParams p)
 
     // The tiles some wave of this workgroup needs, as a list in LDS (build_tile_list): built once per pass of
     // kTileListCap tiles, so the loop below never chases a class word through memory.
-    auto build_list = [&](int c0, int c1, bool have_first, uint32_t w_first) -> int {
+    auto build_list = [&](int c0, int c1, bool have_first, uint32_t w_first) __attribute__((always_inline)) -> int {
         return build_tile_list(p, qb, c0, c1, NT, have_first, w_first, s_list, s_wave_cnt);
     };
     // entry i of the current chunk; without a mask every tile is needed and every class is ZERO
-    auto list_entry = [&](int c0, int i) -> uint32_t {
+    auto list_entry = [&](int c0, int i) __attribute__((always_inline)) -> uint32_t {
         if constexpr (HAS_MASK) return s_list[i];
         else return (uint32_t)(c0 + i) << 8 | 0x55u;
     };
@@ -717,7 +717,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         k_dst[j] = (uint32_t)((r * LDK + cc * 8) * 2);
         v_dst[j] = (uint32_t)((NBUF * BN * LDK + r * LDV + cc * 8) * 2);
     }
-    auto fetch = [&](int t) {
+    auto fetch = [&](int t) __attribute__((always_inline)) {
         const uint32_t slab = (uint32_t)t * (uint32_t)(BN * D * 2); // uniform; part of the checked offset
 #pragma unroll
         for (int j = 0; j < LPT; ++j) {
@@ -725,7 +725,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
             vstage[j] = __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(Vbuf, src_off[j] + slab, 0, 0));
         }
     };
-    auto commit = [&](int buf) {
+    auto commit = [&](int buf) __attribute__((always_inline)) {
         char *base = reinterpret_cast<char *>(smem);
 #pragma unroll
         for (int j = 0; j < LPT; ++j) {
@@ -756,7 +756,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     const int4v Kdesc = raw_descriptor(Kb, (uint32_t)ctx * (uint32_t)(D * 2)), Vdesc = raw_descriptor(Vb, (uint32_t)ctx * (uint32_t)(D * 2));
     typedef __attribute__((address_space(3))) _Float16 *lds_half_ptr;
     const uint32_t lds_tiles = (uint32_t)(uintptr_t)(lds_half_ptr)smem + (uint32_t)wave_u * 2048u; // this wave's blocks
-    auto dma = [&](int t, int buf) {
+    auto dma = [&](int t, int buf) __attribute__((always_inline)) {
         const uint32_t slab = (uint32_t)t * (uint32_t)(BN * D * 2);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -768,7 +768,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     // at chunk (2c+hf) ^ (qi & 15) — one XOR with a constant per read — and the 64-byte unit dt of a V row at
     // unit dt ^ (row & 3); the rows a lane reads differ by multiples of 8, which leaves row & 3 alone.
     const uint32_t k_swz = (uint32_t)(qi * 256 + (((2 * 0 + hf) ^ (qi & 15)) << 4));
-    auto k_operand = [&](int buf, int c) -> half8 {
+    auto k_operand = [&](int buf, int c) __attribute__((always_inline)) -> half8 {
         if constexpr (DMA) return *reinterpret_cast<const half8 *>(reinterpret_cast<const char *>(smem) + (uint32_t)buf * kTileBytes + (k_swz ^ (uint32_t)(c << 5)));
         else return *reinterpret_cast<const half8 *>(&sK[buf][qi][16 * c + 8 * hf]);
     };
@@ -804,7 +804,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         // All loads of a batch are issued before the first value is used (rows past the prompt read the
         // prompt's last row and are zeroed afterwards): left to the compiler, or with the loads under a branch,
         // a wave waits for one chunk before it requests the next — up to eight memory round trips in a row.
-        auto load_queries = [&](auto i32_tag) {
+        auto load_queries = [&](auto i32_tag) __attribute__((always_inline)) {
             constexpr bool I32 = decltype(i32_tag)::value != 0;
             constexpr int BATCH = I32 && QPL > 1 ? QPL / 2 : QPL; // int32 accumulators: twice the registers
             float4 w[2];
@@ -915,7 +915,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     // per-lane source of the transposing V reads: row 4hf + (lane%16)/4, halfs 16*((lane/16)%2) + 4*(lane%4)
     const int vrow = 4 * hf + ((lane & 15) >> 2), vcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
     const uint32_t v_swz = (uint32_t)(vrow * 256 + ((vrow & 3) << 6) + vcol * 2);
-    auto v_operand = [&](int buf, int row0, int dt) -> half4 { // row0: 16u or 16u + 8
+    auto v_operand = [&](int buf, int row0, int dt) __attribute__((always_inline)) -> half4 { // row0: 16u or 16u + 8
         if constexpr (DMA) return lds_read_tr16(reinterpret_cast<const _Float16 *>(reinterpret_cast<const char *>(smem) + (uint32_t)buf * kTileBytes + kVOff + (uint32_t)(row0 * 256) + (v_swz ^ (uint32_t)(dt << 6))));
         else return lds_read_tr16(&sV[buf][row0 + vrow][32 * dt + vcol]);
     };
@@ -951,7 +951,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         }
         // one tile of the pipeline; the LDS buffer index is a compile-time constant (the loop below is
         // unrolled by two), so every LDS address is a register plus an immediate
-        auto tile_step = [&](int i, auto buf_tag) {
+        auto tile_step = [&](int i, auto buf_tag) __attribute__((always_inline)) {
             constexpr int buf = decltype(buf_tag)::value;
             const int t = (int)(e0 >> 8);
             if constexpr (DMA) { // this wave's part of tile t has landed; tile t+1 (four loads) may still be in flight
@@ -1056,7 +1056,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 // use them, and the first set before the softmax: left to itself the compiler reads each pair
                 // right before its product, and every product waits out an LDS round trip.
                 half4 vst[2][4];
-                auto v_stage = [&](int stage, int dt) {
+                auto v_stage = [&](int stage, int dt) __attribute__((always_inline)) {
 #pragma unroll
                     for (int u = 0; u < 2; ++u) {
                         vst[stage][2 * u] = v_operand(buf, 16 * u, dt);
@@ -1382,7 +1382,7 @@ __global__ __launch_bounds__(1024) void attn_quantize_transpose_kernel(const flo
 #pragma unroll
     for (int w = 1; w < 16; ++w) absmax = fmaxf(absmax, s_red[w]);
     if (tid == 0) out_scale[bs] = absmax / 127.0f;
-    auto quant = [&](float value) -> int {
+    auto quant = [&](float value) __attribute__((always_inline)) -> int {
         const float v = rintf(__fmul_rn(value, 127.0f) / absmax);
         return (v != v) ? 0 : (int)fminf(fmaxf(v, -128.f), 127.f); // NaN -> 0, saturate
     };
