@@ -67,8 +67,9 @@ int validate_desc(const fl_attn_desc *d)
     if (!head_dim_ok(d->size_per_head)) return FL_ATTN_ERR_HEAD_DIM;
     if (d->nsplit < 0 || d->nsplit > kMaxSplits || (d->flags & ~FL_ATTN_FLAG_FAST_PROMPT_QK) != 0) return FL_ATTN_ERR_ARGUMENT;
     if (!(d->softmax_scale >= 0.f) || std::isinf(d->softmax_scale)) return FL_ATTN_ERR_ARGUMENT;
-    // row offsets inside one (b,h) slice of a cache are 32-bit byte offsets in the streaming kernel
-    if ((int64_t)d->total_len * d->size_per_head * (d->dtype == FL_ATTN_F16 ? 2 : 4) > (int64_t)UINT32_MAX) return FL_ATTN_ERR_SHAPE;
+    // row offsets inside one (b,h) slice of a cache are 32-bit byte offsets in the kernels; the prompt-phase kernels
+    // form them for whole 32-row tiles, up to 63 rows past the last one (those rows fail the range check and read as zeros)
+    if (((int64_t)d->total_len + 64) * d->size_per_head * (d->dtype == FL_ATTN_F16 ? 2 : 4) > (int64_t)UINT32_MAX) return FL_ATTN_ERR_SHAPE;
     // the streaming grid is one-dimensional: B*H*splits workgroups must fit the 2^31 limit
     if ((int64_t)d->batch_size * d->head_num > (int64_t)INT32_MAX / kMaxSplits) return FL_ATTN_ERR_SHAPE;
     return FL_ATTN_OK;
