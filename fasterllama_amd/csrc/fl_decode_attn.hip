@@ -535,7 +535,7 @@ int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_str
     if (passes & 2) {
         if (!direct && !fused && !check_hip(dispatch_combine(D, p, bh, stream))) return FL_ATTN_ERR_HIP;
         if (quant) {
-            if (!check_hip(launch(flattn::attn_quantize_transpose_kernel, dim3(desc->batch_size), dim3(1024), stream, p.out,
+            if (!check_hip(launch(flattn::attn_quantize_transpose_kernel, dim3(desc->batch_size), dim3(flattn::kQuantThreads), stream, p.out,
                                   io->out_int8, io->out_scale, desc->head_num, 1, D)))
                 return FL_ATTN_ERR_HIP;
         }
@@ -646,7 +646,7 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
     hipError_t e = desc->dtype == FL_ATTN_F16 ? dispatch_prefill<_Float16>(D, p, stream) : dispatch_prefill<float>(D, p, stream);
     if (!check_hip(e)) return FL_ATTN_ERR_HIP;
     if (quant) {
-        if (!check_hip(launch(flattn::attn_quantize_transpose_kernel, dim3((unsigned)(desc->batch_size * seq_len)), dim3(1024),
+        if (!check_hip(launch(flattn::attn_quantize_transpose_kernel, dim3((unsigned)(desc->batch_size * seq_len)), dim3(flattn::kQuantThreads),
                               stream, p.out, io->out_int8, io->out_scale, desc->head_num, seq_len, D)))
             return FL_ATTN_ERR_HIP;
     }

@@ -1345,42 +1345,50 @@ __global__ __launch_bounds__(kWideWaves * 64) void prefill_attn_wide_kernel(cons
 
 // ---------------------------------------------------------------- INT8 epilogue with transpose
 
-// grid = B*S, block = 1024.  attn [B,H,S,D] float -> out_q [B,S,H*D] int8, out_scale [B,S]
+// grid = B*S, block = kQuantThreads.  attn [B,H,S,D] float -> out_q [B,S,H*D] int8, out_scale [B,S]
 // (launchAttnQuantizedTransposeKernel, decoder_kernels.cu:1179-1255); S == 1 is the decode case.
-__global__ __launch_bounds__(1024) void attn_quantize_transpose_kernel(const float *__restrict__ attn,
-                                                                       int8_t *__restrict__ out_q,
-                                                                       float *__restrict__ out_scale, int H, int S, int D)
+// One small workgroup per token, so that a compute unit has eight tokens in flight: the kernel is one memory
+// round trip, a reduction and a store per token, and its bandwidth is what is in flight (1024-thread workgroups,
+// two per compute unit, reached 3.1 TB/s).
+constexpr int kQuantThreads = 256;
+__global__ __launch_bounds__(kQuantThreads) void attn_quantize_transpose_kernel(const float *__restrict__ attn,
+                                                                                int8_t *__restrict__ out_q,
+                                                                                float *__restrict__ out_scale, int H, int S, int D)
 {
-    __shared__ float s_red[16];
+    constexpr int T = kQuantThreads;
+    __shared__ float s_red[T / 64];
     const int bs = blockIdx.x, tid = threadIdx.x;
     const int b = bs / S, s = bs % S;
     const int HD = H * D;
     const float *x = attn + ((size_t)b * H * S + s) * D; // + h * S * D + d
     // A token of up to 8192 values is read ONCE, four consecutive values per lane and trip, and stays in
     // registers between the absmax reduction and the rounding; longer tokens are read twice.
-    constexpr int KEEP = 2; // float4 per thread held in registers
-    const bool keep = HD <= 1024 * 4 * KEEP && (D & 3) == 0;
+    constexpr int KEEP = 8; // float4 per thread held in registers
+    const bool keep = HD <= T * 4 * KEEP && (D & 3) == 0;
     float4 held[KEEP];
     float absmax = kMaxFloor;
     if (keep) {
+        // every load is issued before the first value is used: chunks past the token's end re-read its last one
+        // (under a branch the compiler waits for each load before it requests the next)
 #pragma unroll
         for (int k = 0; k < KEEP; ++k) {
-            const int e = (tid + k * 1024) * 4;
-            held[k] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (e < HD) {
-                held[k] = *reinterpret_cast<const float4 *>(x + (size_t)(e / D) * S * D + e % D);
+            const int e = min((tid + k * T) * 4, HD - 4);
+            held[k] = *reinterpret_cast<const float4 *>(x + (size_t)(e / D) * S * D + e % D);
+        }
+#pragma unroll
+        for (int k = 0; k < KEEP; ++k) {
+            if ((tid + k * T) * 4 < HD)
                 absmax = fmaxf(fmaxf(absmax, fmaxf(fabsf(held[k].x), fabsf(held[k].y))), fmaxf(fabsf(held[k].z), fabsf(held[k].w)));
-            }
         }
     } else {
-        for (int e = tid; e < HD; e += 1024) absmax = fmaxf(absmax, fabsf(x[(size_t)(e / D) * S * D + e % D]));
+        for (int e = tid; e < HD; e += T) absmax = fmaxf(absmax, fabsf(x[(size_t)(e / D) * S * D + e % D]));
     }
     absmax = wave_max(absmax);
     if ((tid & 63) == 0) s_red[tid >> 6] = absmax;
     __syncthreads();
     absmax = s_red[0];
 #pragma unroll
-    for (int w = 1; w < 16; ++w) absmax = fmaxf(absmax, s_red[w]);
+    for (int w = 1; w < T / 64; ++w) absmax = fmaxf(absmax, s_red[w]);
     if (tid == 0) out_scale[bs] = absmax / 127.0f;
     auto quant = [&](float value) __attribute__((always_inline)) -> int {
         const float v = rintf(__fmul_rn(value, 127.0f) / absmax);
@@ -1389,7 +1397,7 @@ __global__ __launch_bounds__(1024) void attn_quantize_transpose_kernel(const flo
     if (keep) {
 #pragma unroll
         for (int k = 0; k < KEEP; ++k) {
-            const int e = (tid + k * 1024) * 4;
+            const int e = (tid + k * T) * 4;
             if (e < HD) {
                 const uint32_t packed = (uint32_t)(quant(held[k].x) & 0xff) | (uint32_t)(quant(held[k].y) & 0xff) << 8 |
                                         (uint32_t)(quant(held[k].z) & 0xff) << 16 | (uint32_t)(quant(held[k].w) & 0xff) << 24;
@@ -1397,7 +1405,7 @@ __global__ __launch_bounds__(1024) void attn_quantize_transpose_kernel(const flo
             }
         }
     } else {
-        for (int e = tid; e < HD; e += 1024)
+        for (int e = tid; e < HD; e += T)
             out_q[(size_t)bs * HD + e] = (int8_t)quant(x[(size_t)(e / D) * S * D + e % D]);
     }
 }
