@@ -334,9 +334,13 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
     constexpr int VEC = flattn::Vec16<T>::N;
     constexpr int LPR = D / VEC < 64 ? D / VEC : 64;
     constexpr int ROWS = 256 / LPR;
-    const int64_t rows = (int64_t)p.B * p.S * p.H;
-    hipError_t e = launch(flattn::prefill_rope_append_kernel<T, D>, dim3((unsigned)((rows + ROWS - 1) / ROWS)), dim3(256),
-                          stream, p);
+    // lane groups of the append kernel: one per token and four heads for fp16 rows where the head count allows
+    // (B=8,S=1024 step 0.1945 -> 0.1912 ms; FP32 rows, twice the bytes per lane already, gain nothing)
+    const int hpt = std::is_same<T, _Float16>::value && p.H % 4 == 0 ? 4 : 1;
+    const int64_t groups = (int64_t)p.B * p.S * (p.H / hpt);
+    const dim3 agrid((unsigned)((groups + ROWS - 1) / ROWS));
+    hipError_t e = hpt == 4 ? launch(flattn::prefill_rope_append_kernel<T, D, 4>, agrid, dim3(256), stream, p)
+                            : launch(flattn::prefill_rope_append_kernel<T, D, 1>, agrid, dim3(256), stream, p);
     if (e != hipSuccess) return e;
     const unsigned qblocks = (unsigned)((p.S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock);
     if (p.attn_mask && !p.class_table) { // no table of the whole mask at hand: classify the rows of this call

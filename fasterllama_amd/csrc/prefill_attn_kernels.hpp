@@ -44,8 +44,10 @@ struct PrefillParams {
 
 // ---------------------------------------------------------------- RoPE + transpose + append
 
-// One lane-group (LPR lanes) per token-head row; grid covers B*S*H rows, 256 threads per block.
-template <typename T, int D>
+// One lane-group (LPR lanes) per token and HPT consecutive heads; grid covers B*S*H/HPT such groups, 256 threads
+// per block.  The heads of a group share the token's cos/sin chunk, and all their loads are issued before the
+// first value is used, so a lane has 2*HPT independent 16-byte loads in flight.
+template <typename T, int D, int HPT>
 __global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillParams p)
 {
     typedef typename Vec16<T>::type V;
@@ -55,43 +57,65 @@ __global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillP
     constexpr int CPL = CH / LPR;
     constexpr int ROWS = 256 / LPR;
 
-    const int64_t rows = (int64_t)p.B * p.S * p.H;
-    const int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / LPR; // index into [B,S,H]
-    if (row >= rows) return;
+    const int HG = p.H / HPT; // head groups per token (the launcher picks HPT so that it divides H)
+    const int64_t groups = (int64_t)p.B * p.S * HG;
+    const int64_t g = (int64_t)blockIdx.x * ROWS + threadIdx.x / LPR; // index into [B,S,H/HPT]
+    if (g >= groups) return;
     const int lig = threadIdx.x % LPR;
-    const int h = (int)(row % p.H);
-    const int64_t bs = row / p.H;
+    const int h0 = (int)(g % HG) * HPT;
+    const int64_t bs = g / HG;
     const int s = (int)(bs % p.S), b = (int)(bs / p.S);
     const int pos = p.start_pos + s;
     const int rope_row = p.rope_row < 0 ? pos : p.rope_row + s;
     const float *freq = p.freq_cis + (size_t)rope_row * D;
     const bool is_i32 = p.inp_scale != nullptr;
     const float inp_scale = is_i32 ? p.inp_scale[bs] : 0.f;
-    const size_t in_off = (size_t)row * D;
-    const size_t bh = (size_t)b * p.H + h;
-    T *kdst = reinterpret_cast<T *>(p.k_cache) + (bh * p.L + pos) * D;
-    T *vdst = reinterpret_cast<T *>(p.v_cache) + (bh * p.L + pos) * D;
 
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
         const int e0 = (c * LPR + lig) * VEC;
-        float kx[VEC], vx[VEC];
-        load_token_chunk<T, VEC>(p.k_new, in_off + e0, is_i32, inp_scale, is_i32 ? p.wk_scale + h * D + e0 : nullptr, kx);
-        load_token_chunk<T, VEC>(p.v_new, in_off + e0, is_i32, inp_scale, is_i32 ? p.wv_scale + h * D + e0 : nullptr, vx);
-        V kt, vt;
+        float kx[HPT][VEC], vx[HPT][VEC];
+        float4 f[VEC / 4];
 #pragma unroll
-        for (int i = 0; i < VEC; i += 4) {
-            const float4 f = *reinterpret_cast<const float4 *>(freq + e0 + i);
-            float r0, r1, r2, r3;
-            rope_pair(kx[i], kx[i + 1], f.x, f.y, r0, r1);
-            rope_pair(kx[i + 2], kx[i + 3], f.z, f.w, r2, r3);
-            kt[i] = to_storage<T>(r0); kt[i + 1] = to_storage<T>(r1);
-            kt[i + 2] = to_storage<T>(r2); kt[i + 3] = to_storage<T>(r3);
+        for (int i = 0; i < VEC; i += 4) f[i / 4] = *reinterpret_cast<const float4 *>(freq + e0 + i);
+        if (is_i32) { // uniform: one straight run of loads per input format
+#pragma unroll
+            for (int hh = 0; hh < HPT; ++hh) {
+                const size_t in_off = (size_t)(bs * p.H + h0 + hh) * D + e0;
+                load_token_chunk<T, VEC>(p.k_new, in_off, true, inp_scale, p.wk_scale + (h0 + hh) * D + e0, kx[hh]);
+                load_token_chunk<T, VEC>(p.v_new, in_off, true, inp_scale, p.wv_scale + (h0 + hh) * D + e0, vx[hh]);
+            }
+        } else {
+            V kraw[HPT], vraw[HPT];
+#pragma unroll
+            for (int hh = 0; hh < HPT; ++hh) {
+                const size_t in_off = (size_t)(bs * p.H + h0 + hh) * D + e0;
+                kraw[hh] = *reinterpret_cast<const V *>(reinterpret_cast<const T *>(p.k_new) + in_off);
+                vraw[hh] = *reinterpret_cast<const V *>(reinterpret_cast<const T *>(p.v_new) + in_off);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int hh = 0; hh < HPT; ++hh)
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) { kx[hh][i] = (float)kraw[hh][i]; vx[hh][i] = (float)vraw[hh][i]; }
         }
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) vt[i] = to_storage<T>(vx[i]);
-        *reinterpret_cast<V *>(kdst + e0) = kt;
-        *reinterpret_cast<V *>(vdst + e0) = vt;
+        for (int hh = 0; hh < HPT; ++hh) {
+            const size_t bh = (size_t)b * p.H + h0 + hh;
+            V kt, vt;
+#pragma unroll
+            for (int i = 0; i < VEC; i += 4) {
+                float r0, r1, r2, r3;
+                rope_pair(kx[hh][i], kx[hh][i + 1], f[i / 4].x, f[i / 4].y, r0, r1);
+                rope_pair(kx[hh][i + 2], kx[hh][i + 3], f[i / 4].z, f[i / 4].w, r2, r3);
+                kt[i] = to_storage<T>(r0); kt[i + 1] = to_storage<T>(r1);
+                kt[i + 2] = to_storage<T>(r2); kt[i + 3] = to_storage<T>(r3);
+            }
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) vt[i] = to_storage<T>(vx[hh][i]);
+            *reinterpret_cast<V *>(reinterpret_cast<T *>(p.k_cache) + (bh * p.L + pos) * D + e0) = kt;
+            *reinterpret_cast<V *>(reinterpret_cast<T *>(p.v_cache) + (bh * p.L + pos) * D + e0) = vt;
+        }
     }
 }
 
