@@ -334,9 +334,10 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
     constexpr int VEC = flattn::Vec16<T>::N;
     constexpr int LPR = D / VEC < 64 ? D / VEC : 64;
     constexpr int ROWS = 256 / LPR;
-    // lane groups of the append kernel: one per token and four heads for fp16 rows where the head count allows
-    // (B=8,S=1024 step 0.1945 -> 0.1912 ms; FP32 rows, twice the bytes per lane already, gain nothing)
-    const int hpt = std::is_same<T, _Float16>::value && p.H % 4 == 0 ? 4 : 1;
+    // lane groups of the append kernel: one per token and four heads for fp16 inputs where the head count allows
+    // (B=8,S=1024: 49.0 -> 44.2 us; FP32 rows and int32 accumulators, twice the bytes per lane already, gain
+    // nothing or lose: 71.2 -> 74.8 us)
+    const int hpt = std::is_same<T, _Float16>::value && !p.inp_scale && p.H % 4 == 0 ? 4 : 1;
     const int64_t groups = (int64_t)p.B * p.S * (p.H / hpt);
     const dim3 agrid((unsigned)((groups + ROWS - 1) / ROWS));
     hipError_t e = hpt == 4 ? launch(flattn::prefill_rope_append_kernel<T, D, 4>, agrid, dim3(256), stream, p)
