@@ -468,7 +468,21 @@ def calibrate(args) -> int:
                 ms = timed(lambda: ok(lib.fl_calib_stream_read(buf.data_ptr(), nbytes, blocks, nt, sink.data_ptr(), sp)), 20)
                 rows.append({"workgroups": blocks, "loads": "nt" if nt else "plain", "us": round(ms * 1e3, 1),
                              "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)})
-        out.update(bytes=nbytes, pattern="128-bit loads, 8 per lane in flight, one contiguous slice per workgroup", results=rows)
+        # the small configurations: what a launch that only READS 64 / 128 / 256 MiB takes, back to back, each launch
+        # on a different slice of the buffer (nothing cache resident) — the floor for configurations 4 and 2
+        small = []
+        for mib in (64, 128, 256):
+            n = mib << 20
+            slices = nbytes // n
+            state = {"i": 0}
+
+            def one(n=n, slices=slices, state=state):
+                state["i"] = (state["i"] + 1) % slices
+                ok(lib.fl_calib_stream_read(buf.data_ptr() + state["i"] * n, n, 256, 1, sink.data_ptr(), sp))
+            ms = timed(one, 200)
+            small.append({"MiB": mib, "workgroups": 256, "loads": "nt", "us": round(ms * 1e3, 2), "GBps": round(n / (ms * 1e-3) / 1e9, 1)})
+        out.update(bytes=nbytes, pattern="128-bit loads, 8 per lane in flight, one contiguous slice per workgroup", results=rows,
+                   small_launches=small)
     elif args.calib == "mfma":
         cus = torch.cuda.get_device_properties(dev).multi_processor_count
         rows = []
