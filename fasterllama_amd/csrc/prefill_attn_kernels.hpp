@@ -631,18 +631,20 @@ __device__ __forceinline__ float max16(const floatx16 &a)
 // absolute on the output, inside the 2e-3 bar of the fp16 path.  The softmax runs in base 2 like the
 // fp16 decode kernels.
 //
-// The matrix cores need 512 cycles per wave and 32x32 tile at D = 128; the softmax between the two
-// products runs on the vector ALU of the same SIMD at 4 cycles per instruction, so its instruction
-// count per score decides the speed (two waves per SIMD overlap one wave's softmax with the other's
-// MFMAs).  Per score the common tile costs: 1/2 v_max3 (maximum over the raw products; the scale is
+// The matrix cores need 512 cycles per wave and 32x32 tile at D = 128 (768 with the query pair); the
+// softmax between the two products runs on the vector ALU of the same SIMD (4 cycles per instruction,
+// 8 for v_exp_f32), and two or three waves per SIMD overlap one wave's softmax with another's MFMAs —
+// as far as the clock allows: with the whole chip on the matrix cores it drops to 1.7-1.9 GHz, and a
+// vector wave beside a matrix wave hides only about half of its time.  Per score the common tile costs: 1/2 v_max3 (maximum over the raw products; the scale is
 // positive, so it commutes with max), 1 v_fma (s*scale - m), 1 v_exp, 1/2 v_cvt_pk_f16_f32 and
 // 1/2 v_dot2c_f32_f16 (the row sum, taken over the rounded probabilities that are multiplied in).
 // The additive mask and the -inf of keys past the context enter as the initial value of the score
 // accumulator; the output accumulators are rescaled lazily (kLazyMax).
 //
-// Data path: K and V tiles (32 keys) are double-buffered in LDS, row-major with padded rows; loads of
-// tile t+2 are in flight in registers while tile t is multiplied, one barrier per tile.  The first
-// product reads K rows as 128-bit operands (S^T = K Q^T).  The second, O^T = V^T P^T, needs eight
+// Data path: K and V tiles (32 keys) pass through LDS, one barrier per tile.  D = 128: loaded straight
+// into swizzled LDS rows (buffer_load ... lds), three buffers, two tiles ahead; D = 32 / 64: row-major
+// with padded rows, two buffers, the loads of tile t+2 in flight in registers while tile t is multiplied.
+// The first product reads K rows as 128-bit operands (S^T = K Q^T).  The second, O^T = V^T P^T, needs eight
 // keys of one d per lane: ds_read_b64_tr_b16 delivers exactly that from the row-major tile (within
 // 16 lanes, lanes 4j..4j+3 address 16 consecutive halfs of row j; lane i receives element i of rows
 // 0..3), so V is never transposed in memory.  Contraction slots of the second product: a lane-half
