@@ -432,6 +432,7 @@ def calibrate(args) -> int:
     lib.fl_calib_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     lib.fl_calib_mfma.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     lib.fl_calib_empty.argtypes = [C.c_void_p]
+    lib.fl_calib_stream_read_two.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_void_p]
     lib.fl_calib_coexec.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     dev = torch.device("cuda:0")
     stream = torch.cuda.current_stream(dev)
@@ -468,6 +469,10 @@ def calibrate(args) -> int:
                 ms = timed(lambda: ok(lib.fl_calib_stream_read(buf.data_ptr(), nbytes, blocks, nt, sink.data_ptr(), sp)), 20)
                 rows.append({"workgroups": blocks, "loads": "nt" if nt else "plain", "us": round(ms * 1e3, 1),
                              "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)})
+        for blocks in (2048, 8192):  # the decode step's own pattern: K rows and V rows, two streams per workgroup
+            ms = timed(lambda: ok(lib.fl_calib_stream_read_two(buf.data_ptr(), nbytes, blocks, sink.data_ptr(), sp)), 20)
+            rows.append({"workgroups": blocks, "loads": "nt, two streams of 4 loads per lane (K rows, V rows)", "us": round(ms * 1e3, 1),
+                         "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)})
         # the small configurations: what a launch that only READS 64 / 128 / 256 MiB takes, back to back, each launch
         # on a different slice of the buffer (nothing cache resident) — the floor for configurations 4 and 2
         small = []

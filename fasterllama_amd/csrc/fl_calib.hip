@@ -3,6 +3,7 @@
 // the nominal peak alone.  Nothing here is part of the attention path; libfl_decode_attn.so does not link it.
 //   fl_calib_stream_read   128-bit coalesced streaming read of a buffer, plain or non-temporal loads,
 //                          one workgroup per contiguous slice (the access pattern of the decode step)
+//   fl_calib_stream_read_two  the same bytes as two streams per workgroup, half the buffer apart (K rows and V rows)
 //   fl_calib_empty         a kernel that does nothing (launch cadence of back-to-back dependent launches)
 //   fl_calib_mfma_f16/f32  register-only loops of v_mfma_f32_32x32x16_f16 / v_mfma_f32_32x32x2_f32
 //   fl_calib_coexec        one wave of matrix work and one wave of vector (fma + exp2) work per SIMD, each alone
@@ -32,6 +33,26 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const char *src, uint3
         for (int u = 0; u < 8; ++u) acc ^= v[u];
     }
     if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[0] = 1.f; // keeps the loads alive
+}
+
+// The decode step's pattern: a workgroup streams TWO slices (its K rows and its V rows, half the buffer apart),
+// four 16-byte non-temporal loads per lane in flight on each.
+__global__ __launch_bounds__(256) void stream_read_two_kernel(const char *src, uint32_t bytes_per_block, size_t second, float *sink)
+{
+    const char *base = src + (size_t)blockIdx.x * bytes_per_block;
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(base), 0, (int)bytes_per_block, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(base + second), 0, (int)bytes_per_block, 0x00020000);
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    for (uint32_t off = threadIdx.x * 16u; off < bytes_per_block; off += 4u * 4096u) {
+        u32x4 a[4], b[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) a[u] = __builtin_amdgcn_raw_buffer_load_b128(ra, off, (uint32_t)u * 4096u, 2);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) b[u] = __builtin_amdgcn_raw_buffer_load_b128(rb, off, (uint32_t)u * 4096u, 2);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc ^= a[u] ^ b[u];
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[0] = 1.f;
 }
 
 __global__ void empty_kernel() {}
@@ -157,6 +178,16 @@ int fl_calib_stream_read(const void *src, size_t bytes, int blocks, int nontempo
         hipLaunchKernelGGL(stream_read_kernel<2>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const char *>(src), per_block, sink);
     else
         hipLaunchKernelGGL(stream_read_kernel<0>, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const char *>(src), per_block, sink);
+    return (int)hipGetLastError();
+}
+
+// Reads `bytes` from src once as two streams: workgroup i reads slice i of the first half and slice i of the second
+// half, alternately.  bytes must be a multiple of blocks * 32768.
+int fl_calib_stream_read_two(const void *src, size_t bytes, int blocks, float *sink, void *stream)
+{
+    if (!src || !sink || blocks <= 0 || bytes % ((size_t)blocks * 32768u) != 0 || bytes / 2 / blocks > 0x7fffffffu) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(stream_read_two_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const char *>(src), (uint32_t)(bytes / 2 / blocks), bytes / 2, sink);
     return (int)hipGetLastError();
 }
 
