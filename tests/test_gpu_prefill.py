@@ -298,6 +298,42 @@ def test_prefill_llama7b_shape(gpu):
     assert_out_close(out, want, "f16", "7B prompt 512")
 
 
+@pytest.mark.parametrize("fast", [False, True])
+def test_prefill_benchmark_shape_full_size(gpu, fast):
+    """The prompt-phase benchmark shape at full size (B=8, H=32, S=1024, D=128, fp16 caches, the reference driver's
+    causal mask, tile classes from the persistent table).  Heads are independent, so the oracle runs on a sample of
+    (b,h) pairs cut out of the same inputs; their output rows and cache rows are checked, the caches bit for bit."""
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    B, H, D, L, S = 8, 32, 128, 1024, 1024
+    dev = gpu
+    g = torch.Generator(device="cpu").manual_seed(77)
+    q = torch.randn(B, S, H, D, generator=g).half()
+    k = torch.randn(B, S, H, D, generator=g).half()
+    v = torch.randn(B, S, H, D, generator=g).half()
+    f = synth.freq_cis_table(L, D)
+    mask = causal_mask(L, -FMAX)
+    op = PrefillAttention(B, H, D, L, S, torch.float16, device=dev, fast_qk=fast)
+    md = torch.from_numpy(mask).to(dev)
+    table = op.classify_mask(md)
+    kc = torch.full((B, H, L, D), float("nan"), dtype=torch.float16, device=dev)
+    vc = torch.full((B, H, L, D), float("nan"), dtype=torch.float16, device=dev)
+    out = op.prefill(q.to(dev), k.to(dev), v.to(dev), kc, vc, torch.from_numpy(f).to(dev), attn_mask=md, mask_tile_classes=table)
+    torch.cuda.synchronize()
+    assert not torch.isnan(out).any() and not torch.isnan(kc).any() and not torch.isnan(vc).any()
+    for b, h in ((0, 0), (3, 17), (7, 31), (4, 5)):
+        qs, ks, vs = (x[b:b + 1, :, h:h + 1, :].contiguous().numpy() for x in (q, k, v))
+        kr = np.full((1, 1, L, D), np.nan, np.float16)
+        vr = np.full((1, 1, L, D), np.nan, np.float16)
+        want = ref.prefill_attn(qs, ks, vs, kr, vr, f, start_pos=0, attn_mask=mask, acc_double=True, threads=16)
+        assert_cache_bit_exact(kc[b:b + 1, h:h + 1].cpu().numpy(), kr, f"k_cache ({b},{h})")
+        assert_cache_bit_exact(vc[b:b + 1, h:h + 1].cpu().numpy(), vr, f"v_cache ({b},{h})")
+        if not fast:  # the single-fp16-query product is judged on ordinary data elsewhere; here it must stay close
+            assert_out_close(out[b:b + 1, h:h + 1].cpu().numpy(), want, "f16", f"benchmark shape, pair ({b},{h})")
+        else:
+            assert np.abs(out[b:b + 1, h:h + 1].cpu().numpy() - want).max() <= 2e-3
+
+
 def test_prefill_then_decode_steps_agree_with_oracle_sequence(gpu):
     """Prompt of 70 tokens, then 5 decode steps on the same caches: every step against the oracle, caches
     bit-identical at the end (the two paths write the same rows the same way)."""
