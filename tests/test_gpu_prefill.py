@@ -298,14 +298,16 @@ def test_prefill_llama7b_shape(gpu):
     assert_out_close(out, want, "f16", "7B prompt 512")
 
 
-@pytest.mark.parametrize("fast", [False, True])
-def test_prefill_benchmark_shape_full_size(gpu, fast):
-    """The prompt-phase benchmark shape at full size (B=8, H=32, S=1024, D=128, fp16 caches, the reference driver's
-    causal mask, tile classes from the persistent table).  Heads are independent, so the oracle runs on a sample of
+@pytest.mark.parametrize("B,S,pairs,fast", [(8, 1024, ((0, 0), (3, 17), (7, 31), (4, 5)), False),
+                                            (8, 1024, ((0, 0), (3, 17), (7, 31), (4, 5)), True),
+                                            (1, 4096, ((0, 0), (0, 21)), False)])
+def test_prefill_benchmark_shape_full_size(gpu, B, S, pairs, fast):
+    """The prompt-phase benchmark shapes at full size (B=8, S=1024 and B=1, S=4096; H=32, D=128, fp16 caches, the
+    reference driver's causal mask, tile classes from the persistent table).  Heads are independent, so the oracle runs on a sample of
     (b,h) pairs cut out of the same inputs; their output rows and cache rows are checked, the caches bit for bit."""
     import torch
     from fasterllama_amd.decode_attn import PrefillAttention
-    B, H, D, L, S = 8, 32, 128, 1024, 1024
+    H, D, L = 32, 128, S
     dev = gpu
     g = torch.Generator(device="cpu").manual_seed(77)
     q = torch.randn(B, S, H, D, generator=g).half()
@@ -321,7 +323,7 @@ def test_prefill_benchmark_shape_full_size(gpu, fast):
     out = op.prefill(q.to(dev), k.to(dev), v.to(dev), kc, vc, torch.from_numpy(f).to(dev), attn_mask=md, mask_tile_classes=table)
     torch.cuda.synchronize()
     assert not torch.isnan(out).any() and not torch.isnan(kc).any() and not torch.isnan(vc).any()
-    for b, h in ((0, 0), (3, 17), (7, 31), (4, 5)):
+    for b, h in pairs:
         qs, ks, vs = (x[b:b + 1, :, h:h + 1, :].contiguous().numpy() for x in (q, k, v))
         kr = np.full((1, 1, L, D), np.nan, np.float16)
         vr = np.full((1, 1, L, D), np.nan, np.float16)
