@@ -52,3 +52,36 @@ def test_noalloc_rejects_what_does_not_fit(gpu):
     io.workspace, io.workspace_bytes = None, 0
     st = op.launch_noalloc(io)
     assert st == capi.FL_ATTN_ERR_SCRATCH_LIMIT and "scratch" in capi.strerror(st)
+
+
+def test_noalloc_call_can_be_captured_in_a_hip_graph(gpu):
+    """Callers under graph capture are who the entry point is for: after one eager call on the device (which looks
+    up the scratch array's address) the call only enqueues kernels.  Replays, interleaved with unrelated eager work,
+    reproduce the eager result bit for bit, with a split context (partials and arrival counters in the scratch array)."""
+    import torch
+    from fasterllama_amd.decode_attn import DecodeAttention
+    B, H, D, L, P = 2, 16, 128, 4096, 3000
+    c = Case(B, H, D, L, "f16", start_pos=P)
+    t = lambda a: torch.from_numpy(a).to(gpu)
+    op = DecodeAttention(B, H, D, L, torch.float16, nsplit=8, device=gpu)
+    q, k, v, kc, vc, f = (t(a) for a in (c.q, c.k_new, c.v_new, c.k_cache, c.v_cache, c.freq))
+    out = torch.zeros(B, H * D, device=gpu)
+    io = op.make_io(q, k, v, kc, vc, f, out, start_pos=P)
+    io.workspace, io.workspace_bytes = None, 0
+    assert op.launch_noalloc(io) == 0
+    torch.cuda.synchronize()
+    eager = out.clone()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream(device=gpu)
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            assert op.launch_noalloc(io, stream=torch.cuda.current_stream(gpu)) == 0
+    torch.cuda.synchronize()
+    for rep in range(3):
+        out.fill_(float("nan"))
+        _ = (torch.randn(1 << 20, device=gpu) * 2).sum().item()  # unrelated eager work + sync
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep}"
+    want64 = c.run_oracle(acc_double=True, threads=16)[0]
+    assert_out_close(out.cpu().numpy(), want64, "f16", "noalloc graph replay", head_dim=D)
