@@ -121,24 +121,61 @@ __global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillP
 
 // ---------------------------------------------------------------- dense attention on MFMA
 
-// RoPE(q) for N consecutive head dims d0.. of one prompt token, in FP32: the attention kernels
-// rotate their own queries while they load them (decoder_kernels.cu:449-458), so the rotated
-// queries never travel through memory.  `token` indexes [B,S], `row` is the table row.
-// I32: 1 / 0 when the caller has already branched on the input format (int32 accumulators or not), -1 to test here.
-template <typename T, int N, int I32 = -1>
-__device__ __forceinline__ void rotated_query_chunk(const PrefillParams &p, int D, int64_t token, int h, int d0, int row,
-                                                    float (&out)[N])
+// RoPE(q) for the head dims one lane of the FP32-MFMA kernels owns — dims d_first + 8c + (0..3) for c < NC — of one
+// prompt token, in FP32: the attention kernels rotate their own queries while they load them
+// (decoder_kernels.cu:449-458), so the rotated queries never travel through memory.  `token` indexes [B,S],
+// `row` is the table row.  The input format (int32 accumulators or not) is branched on ONCE and all loads of a
+// batch are issued before the first value is used: with the branch and the use inside the loop over chunks a
+// wave waited out one memory round trip per chunk, sixteen in a row at D = 128.
+template <typename T, int NC>
+__device__ __forceinline__ void rotated_query_lane(const PrefillParams &p, int D, int64_t token, int h, int d_first, int row,
+                                                   float (&out)[NC][4])
 {
-    const bool is_i32 = I32 < 0 ? p.inp_scale != nullptr : I32 != 0;
-    float x[N];
-    load_token_chunk<T, N>(p.q, (size_t)(token * p.H + h) * D + d0, is_i32, is_i32 ? p.inp_scale[token] : 0.f,
-                           is_i32 ? p.wq_scale + h * D + d0 : nullptr, x);
-    const float *freq = p.freq_cis + (size_t)row * D + d0;
+    const size_t q_off = (size_t)(token * p.H + h) * D + d_first;
+    const float *freq = p.freq_cis + (size_t)row * D + d_first;
+    auto rotate = [&](const float (&x)[4], const float4 &f, float (&o)[4]) __attribute__((always_inline)) {
+        rope_pair(x[0], x[1], f.x, f.y, o[0], o[1]);
+        rope_pair(x[2], x[3], f.z, f.w, o[2], o[3]);
+    };
+    if (p.inp_scale != nullptr) {
+        const float sc = p.inp_scale[token];
+        const int32_t *qi = reinterpret_cast<const int32_t *>(p.q) + q_off;
+        const float *w = p.wq_scale + h * D + d_first;
+        constexpr int BATCH = NC > 8 ? 8 : NC;
 #pragma unroll
-    for (int i = 0; i < N; i += 4) {
-        const float4 f = *reinterpret_cast<const float4 *>(freq + i);
-        rope_pair(x[i], x[i + 1], f.x, f.y, out[i], out[i + 1]);
-        rope_pair(x[i + 2], x[i + 3], f.z, f.w, out[i + 2], out[i + 3]);
+        for (int c0 = 0; c0 < NC; c0 += BATCH) {
+            int4 a[BATCH];
+            float4 ws[BATCH], f[BATCH];
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                a[j] = *reinterpret_cast<const int4 *>(qi + 8 * (c0 + j));
+                ws[j] = *reinterpret_cast<const float4 *>(w + 8 * (c0 + j));
+                f[j] = *reinterpret_cast<const float4 *>(freq + 8 * (c0 + j));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) { // decoder_kernels.cu:449-452
+                const float x[4] = {__fmul_rn(__fmul_rn((float)a[j].x, sc), ws[j].x), __fmul_rn(__fmul_rn((float)a[j].y, sc), ws[j].y),
+                                    __fmul_rn(__fmul_rn((float)a[j].z, sc), ws[j].z), __fmul_rn(__fmul_rn((float)a[j].w, sc), ws[j].w)};
+                rotate(x, f[j], out[c0 + j]);
+            }
+        }
+    } else {
+        typedef T vec4 __attribute__((ext_vector_type(4)));
+        const T *qt = reinterpret_cast<const T *>(p.q) + q_off;
+        vec4 a[NC];
+        float4 f[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            a[c] = *reinterpret_cast<const vec4 *>(qt + 8 * c);
+            f[c] = *reinterpret_cast<const float4 *>(freq + 8 * c);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const float x[4] = {(float)a[c][0], (float)a[c][1], (float)a[c][2], (float)a[c][3]};
+            rotate(x, f[c], out[c]);
+        }
     }
 }
 
@@ -342,11 +379,10 @@ void prefill_attn_kernel(const PrefillParams p)
     {
         const int64_t token = (int64_t)(bh / p.H) * S + (q_ok ? q_row : 0);
         const int row = (p.rope_row < 0 ? P : p.rope_row) + (q_ok ? q_row : 0);
+        rotated_query_lane<T, NC>(p, D, token, bh % p.H, 4 * hf, row, qreg);
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            rotated_query_chunk<T, 4>(p, D, token, bh % p.H, 8 * c + 4 * hf, row, qreg[c]);
+        for (int c = 0; c < NC; ++c)
             if (!q_ok) qreg[c][0] = qreg[c][1] = qreg[c][2] = qreg[c][3] = 0.f;
-        }
     }
 
     floatx16 ot[NDT];
@@ -1245,11 +1281,10 @@ __global__ __launch_bounds__(kWideWaves * 64) void prefill_attn_wide_kernel(cons
     {
         const int64_t token = (int64_t)(bh / p.H) * S + (q_ok ? q_row : 0);
         const int row = (p.rope_row < 0 ? P : p.rope_row) + (q_ok ? q_row : 0);
+        rotated_query_lane<T, NC>(p, D, token, bh % p.H, d_wave + 4 * hf, row, qreg);
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            rotated_query_chunk<T, 4>(p, D, token, bh % p.H, d_wave + 8 * c + 4 * hf, row, qreg[c]);
+        for (int c = 0; c < NC; ++c)
             if (!q_ok) qreg[c][0] = qreg[c][1] = qreg[c][2] = qreg[c][3] = 0.f;
-        }
     }
 
     floatx16 ot[NDT];
