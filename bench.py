@@ -60,19 +60,28 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 matrix rate (fp16 
 
 
 def bench_prefill(args) -> int:
-    """One step = RoPE + append + dense attention of S new tokens per sequence (prompt phase)."""
+    """Prints the JSON line of one prompt-phase workload."""
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    print(json.dumps(measure_prefill(args, args.workload, min(args.steps, 50), min(args.warmup, 5), args.repeats,
+                                     cpu=not args.no_cpu)), flush=True)
+    return 0
+
+
+def measure_prefill(args, workload, steps, warm, repeats, cpu=False) -> dict:
+    """One step = RoPE + append + dense attention of S new tokens per sequence (prompt phase).  Returns the
+    workload's JSON object."""
     import numpy as np
     import torch
 
     from fasterllama_amd import capi, synth
     from fasterllama_amd.decode_attn import PrefillAttention
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        return 3
     capi.load()
     dev = torch.device("cuda:0")
-    w = PREFILL_WORKLOADS[args.workload]
+    w = PREFILL_WORKLOADS[workload]
     B, H, D, S, P, L = w["B"], w["H"], w["D"], w["S"], w["P"], w["L"]
     np_dt = np.float16 if w["dtype"] == "f16" else np.float32
     t_dt = torch.float16 if w["dtype"] == "f16" else torch.float32
@@ -100,7 +109,7 @@ def bench_prefill(args) -> int:
     if args.segment == "int32-int8":
         # the segment as OpenDecoder::forward feeds it: int32 accumulators + scales in, per-token INT8 + scale out, no
         # float output (the float result passes through the workspace to the quantisation kernel)
-        args.no_cpu = True
+        cpu = False
         rng = np.random.default_rng(args.seed)
         q, k, v = (torch.from_numpy(rng.integers(-20000, 20000, (B, S, H, D), dtype=np.int32)).to(dev) for _ in range(3))
         extra = dict(
@@ -121,10 +130,9 @@ def bench_prefill(args) -> int:
             if st != 0:
                 raise capi.FlAttnError(st, capi.strerror(st))
 
-    steps, warm = min(args.steps, 50), min(args.warmup, 5)
     run(warm)
     torch.cuda.synchronize()
-    ms, ms_all = time_region(torch, stream, run, steps, args.repeats)
+    ms, ms_all = time_region(torch, stream, run, steps, repeats)
     dense_flops = 4.0 * B * H * S * (P + S) * D  # every query against every key
     # FLOPs the kernels execute: 32x32 tiles whose mask entries are all <= -1e30 are dropped (their weights
     # are exactly 0); every other tile is multiplied.
@@ -140,8 +148,8 @@ def bench_prefill(args) -> int:
     peak = MFMA_FP16_PEAK_TFLOPS if w["dtype"] == "f16" else MFMA_FP32_PEAK_TFLOPS
 
     max_err = None
-    cpu = None
-    if not args.no_cpu:
+    cpu_leg = None
+    if cpu:
         from oracle import ref  # checker / baseline only
         nb = 1
         kc_s = np.zeros((nb, H, L, D), np_dt)
@@ -152,17 +160,19 @@ def bench_prefill(args) -> int:
                                 attn_mask=None if args.prefill_mask == "none" else mask_h, threads=nthreads)
         dt_cpu = time.perf_counter() - t1
         max_err = float(np.abs(out[:nb].cpu().numpy() - want).max())
-        cpu = {"value": round(4.0 * nb * H * S * (P + S) * D / dt_cpu / 1e12, 5), "unit": "TFLOP/s (dense count)", "cores": nthreads,
+        cpu_leg = {"value": round(4.0 * nb * H * S * (P + S) * D / dt_cpu / 1e12, 5), "unit": "TFLOP/s (dense count)", "cores": nthreads,
                "kind": "port", "sample": f"first {nb} of {B} sequences, scalar oracle with OpenMP over heads, {dt_cpu:.2f} s",
                "gpu_vs_oracle_max_abs_err": max_err}
-    print(json.dumps({
-        "metric": f"prompt-phase attention TFLOP/s, {args.workload}", "value": round(tflops, 2), "unit": "TFLOP/s",
-        "n_gpus": 1, "steps": steps, "warmup": warm, "repeats": args.repeats, "ms_per_step": round(ms, 5),
+    del kc, vc, q, k, v, out, io, op
+    torch.cuda.empty_cache()
+    return {
+        "metric": f"prompt-phase attention TFLOP/s, {workload}", "value": round(tflops, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": steps, "warmup": warm, "repeats": repeats, "ms_per_step": round(ms, 5),
         "ms_per_step_all_regions": [round(x, 5) for x in ms_all], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 MFMA, f32 accumulate (f16 storage)" if w["dtype"] == "f16" else "f32 MFMA",
         "data": "synthetic (seeded splitmix64 + Box-Muller N(0,1), seed %d)" % args.seed,
-        "config": {"workload": f"{args.workload}: B={B} H={H} D={D} S={S} start_pos={P} L={L} {w['dtype']} KV cache, "
+        "config": {"workload": f"{workload}: B={B} H={H} D={D} S={S} start_pos={P} L={L} {w['dtype']} KV cache, "
                                + {"causal": "causal additive mask, -FLT_MAX above the diagonal",
                                   "causal-1e5": "causal additive mask, -1e5 above the diagonal",
                                   "block-causal": "additive mask, causal over blocks of 128 tokens, -FLT_MAX above",
@@ -171,12 +181,38 @@ def bench_prefill(args) -> int:
                                + (", mask tiles classified once per mask" if table is not None else "")
                                + (", int32 accumulators in, INT8 + scale out" if args.segment == "int32-int8" else ""),
                    "flops_per_step": flops, "dense_flops_per_step": dense_flops,
+                   "dense_tflops": round(dense_flops / (ms * 1e-3) / 1e12, 2),
                    "tokens_per_s": round(B * S / (ms * 1e-3), 1)},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(tflops / peak, 4), "traffic": None,
                      "kernel": "prefill_attn_kernel (+ prefill_rope_append_kernel, same step)"},
-        "cpu_baseline": cpu}), flush=True)
-    return 0
+        "cpu_baseline": cpu_leg}
+
+
+def prefill_summary(line):
+    """The figures of one prompt-phase workload as they appear under other_configs."""
+    return {"workload": line["config"]["workload"], "ms_per_step": line["ms_per_step"],
+            "tflops_executed": line["value"], "tflops_dense_count": line["config"]["dense_tflops"],
+            "mfma_peak_tflops": line["roofline"]["peak"], "frac_of_mfma_peak": line["roofline"]["frac"],
+            "note": "whole step: append kernel + attention kernel; executed = tiles the causal mask leaves (-FLT_MAX tiles "
+                    "are exact zeros and dropped), dense = every query against every key",
+            "ms_per_step_all_regions": line["ms_per_step_all_regions"]}
+
+
+def opendecoder_loop(B, H, D, L, P, layers, steps):
+    """OpenDecoder::forward in the reference driver's layer loop (initialize(param[layer], buf) before every
+    forward), timed by the C++ program fasterllama_amd/lib/open_decoder_bench; its JSON object, or an error note."""
+    import subprocess
+
+    from fasterllama_amd import build
+    exe = build.outputs("cxxbench")
+    if not os.path.exists(exe):
+        return {"error": f"{exe} has not been built (python -m fasterllama_amd.build cxxbench)"}
+    res = subprocess.run([exe] + [str(x) for x in (B, H, D, L, P, layers, steps)], stdout=subprocess.PIPE,
+                         stderr=subprocess.PIPE, text=True, timeout=300)
+    if res.returncode != 0:
+        return {"error": f"open_decoder_bench exited with {res.returncode}: {res.stderr.strip()[-300:]}"}
+    return json.loads(res.stdout.strip().splitlines()[-1])
 
 def measured_traffic(workload: str, mask: str):
     """HBM bytes per launch of the streaming kernel for this workload, as measured with rocprofv3 --pmc
@@ -561,6 +597,9 @@ def main() -> int:
     ap.add_argument("--two-launches", action="store_true",
                     help="decode workloads: skip fl_decode_attn_workspace_init, so that a split context is merged "
                          "by a second launch instead of inside the streaming kernel")
+    ap.add_argument("--opendecoder-loop", action="store_true",
+                    help="time OpenDecoder::forward in the reference driver's layer loop at the workload's shape "
+                         "(fasterllama_amd/lib/open_decoder_bench), print its JSON object and exit")
     ap.add_argument("--segment", default="attention", choices=["attention", "int32-int8"],
                     help="attention: q/k/v in the cache dtype -> float output (the headline metric). "
                          "int32-int8: the whole reference segment, int32 GEMM accumulators + scales in, "
@@ -594,6 +633,13 @@ def main() -> int:
         return 3
     if args.calib:
         return calibrate(args)
+    if args.opendecoder_loop:
+        w = WORKLOADS.get(args.workload)
+        if w is None or w.get("ragged") or w["dtype"] != "f16":
+            print("bench.py: --opendecoder-loop needs a uniform fp16 decode workload", file=sys.stderr)
+            return 2
+        print(json.dumps(opendecoder_loop(w["B"], w["H"], w["D"], w["L"], w["ctx"] - 1, w["copies"], 20)), flush=True)
+        return 0
     if args.workload in PREFILL_WORKLOADS:
         return bench_prefill(args)
     capi.load()  # fails loudly when the HIP library is missing
@@ -616,6 +662,15 @@ def main() -> int:
                                 ("cfg5", "cfg5", "none"), ("cfg3_causal_mask", "cfg3", "causal"),
                                 ("cfg3_strict_mask", "cfg3", "strict")):
             others[key] = summary(measure_decode(name, args, o_steps, max(3, args.warmup // 2), o_rep, mask=mask))
+        # the prompt phase of the same block (matrix-core bound: another roofline), reference driver's causal mask
+        saved = (args.prefill_mask, args.prefill_fast_qk, args.prefill_classify_per_call)
+        args.prefill_mask, args.prefill_fast_qk, args.prefill_classify_per_call = "causal", False, False
+        for name in ("prefill_7b_b8_s1024", "prefill_7b_b8_s1024_f32", "prefill_7b_b1_s4096"):
+            others[name] = prefill_summary(measure_prefill(args, name, 20, 3, 3))
+        args.prefill_mask, args.prefill_fast_qk, args.prefill_classify_per_call = saved
+        # OpenDecoder::forward under the reference driver's call pattern, at the small (B=1, ctx 4096) and the headline shape
+        others["opendecoder_loop_cfg4"] = opendecoder_loop(1, 32, 128, 4096, 4095, 12, 20)
+        others["opendecoder_loop_cfg3"] = opendecoder_loop(64, 32, 128, 2048, 2047, 1, 20)
 
     line = {
         "metric": "decode-attn us/step + HBM GB/s (% peak), LLaMA2-7B heads b=64 ctx=2048 fp16"

@@ -10,6 +10,7 @@ Targets
     calib   fasterllama_amd/lib/libfl_calib.so         measurement-only kernels of bench.py --calib
     oracle  oracle/libfl_ref.so                        CPU checker (test infrastructure)
     cpptest tests/cpp/open_decoder_check               C++ drop-in test driver
+    cxxbench fasterllama_amd/lib/open_decoder_bench    times OpenDecoder::forward in the reference driver's layer loop
     sanitize (by name only) oracle + C-ABI host logic built with ASan/UBSan and run on the CPU
 """
 from __future__ import annotations
@@ -47,6 +48,8 @@ def sources(name: str) -> list[str]:
         "oracle": [os.path.join(ROOT, "oracle", "fl_ref_decode_attn.c"), os.path.join(ROOT, "oracle", "Makefile")],
         "cpptest": [os.path.join(ROOT, "tests", "cpp", "open_decoder_check.cpp"), os.path.join(CSRC, "open_decoder.h"),
                     os.path.join(ROOT, "include", "fl_decode_attn.h")],
+        "cxxbench": [os.path.join(CSRC, "open_decoder_bench.cpp"), os.path.join(CSRC, "open_decoder.h"),
+                     os.path.join(ROOT, "include", "fl_decode_attn.h")],
     }[name]
 
 
@@ -58,6 +61,7 @@ def outputs(name: str) -> str:
         "calib": os.path.join(LIB, "libfl_calib.so"),
         "oracle": os.path.join(ROOT, "oracle", "libfl_ref.so"),
         "cpptest": os.path.join(ROOT, "tests", "cpp", "open_decoder_check"),
+        "cxxbench": os.path.join(LIB, "open_decoder_bench"),
     }[name]
 
 
@@ -160,6 +164,14 @@ def build_cpptest() -> str:
     return _built("cpptest")
 
 
+def build_cxxbench() -> str:
+    out = outputs("cxxbench")
+    _run([hipcc(), "-O2", "-std=c++17", "-Wall", "-I", os.path.join(ROOT, "include"), "-I", CSRC, "-o", out,
+          os.path.join(CSRC, "open_decoder_bench.cpp"), "-L", LIB, "-lflopendecoder", "-lfl_decode_attn",
+          f"-Wl,-rpath,{LIB}", "-Wl,-rpath,$ORIGIN"])
+    return _built("cxxbench")
+
+
 def run_sanitizers() -> None:
     """Host code under AddressSanitizer + UndefinedBehaviorSanitizer, built and RUN here (no GPU involved):
     the CPU oracle with its driver (`make -C oracle asan`), and the host pass of the C-ABI library with
@@ -183,6 +195,7 @@ TARGETS = {
     "calib": build_calib,
     "oracle": build_oracle,
     "cpptest": build_cpptest,
+    "cxxbench": build_cxxbench,
     "sanitize": run_sanitizers,
 }
 DEFAULT_TARGETS = [t for t in TARGETS if t != "sanitize"]  # the sanitizer run is asked for by name (and by the CPU tests)

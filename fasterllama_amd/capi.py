@@ -27,6 +27,7 @@ FL_ATTN_ERR_HIP = -7
 FL_ATTN_ERR_ALIGNMENT = -8
 FL_ATTN_ERR_ARGUMENT = -9
 FL_ATTN_ERR_SCRATCH_LIMIT = -10
+FL_ATTN_ERR_STRUCT_SIZE = -11
 FL_ATTN_IO_WORKSPACE_READY = 1
 FL_ATTN_NOALLOC_SCRATCH_BYTES = 16 << 20
 
@@ -51,7 +52,9 @@ EXPORTED_SYMBOLS = (
 
 
 class AttnDesc(C.Structure):
+    """fl_attn_desc; AttnDesc(B, H, D, L, dtype, nsplit, softmax_scale, flags) fills struct_size itself."""
     _fields_ = [
+        ("struct_size", C.c_uint32),
         ("batch_size", C.c_int32),
         ("head_num", C.c_int32),
         ("size_per_head", C.c_int32),
@@ -62,9 +65,13 @@ class AttnDesc(C.Structure):
         ("flags", C.c_int32),
     ]
 
+    def __init__(self, *args, **kw):
+        super().__init__(C.sizeof(AttnDesc), *args, **kw)
+
 
 class AttnIO(C.Structure):
     _fields_ = [
+        ("struct_size", C.c_uint32),
         ("q", C.c_void_p),
         ("k_new", C.c_void_p),
         ("v_new", C.c_void_p),
@@ -89,6 +96,10 @@ class AttnIO(C.Structure):
         ("out_scale", C.c_void_p),
         ("mask_tile_classes", C.c_void_p),
     ]
+
+    def __init__(self, **kw):
+        super().__init__(**kw)
+        self.struct_size = C.sizeof(AttnIO)
 
 
 class AttnPlan(C.Structure):

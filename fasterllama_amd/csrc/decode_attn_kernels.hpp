@@ -210,7 +210,8 @@ constexpr int kCombineMaxSplits = 1024;
 template <int D>
 struct CombineShared {
     static constexpr int TPG = D / 4 < kCombineThreads ? D / 4 : kCombineThreads; // threads per split-group
-    static constexpr int SG = kCombineThreads / TPG;                             // split-groups
+    static constexpr int SG = kCombineThreads / TPG;                             // split-groups (whole ones: at D = 96 the
+                                                                                 // last 16 threads of the workgroup own none)
     float w[kCombineMaxSplits];
     float red[2][kCombineThreads / 64];
     float4 acc[SG][D / 4];
@@ -262,6 +263,7 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
     // the first 256 splits and the first four partial rows of this thread's split-group — so that the
     // merge waits for memory once, not once per phase.  The arithmetic and its order do not depend on it.
     const int sg = tid / TPG, t = tid % TPG;
+    const bool in_group = SG * TPG == kCombineThreads || sg < SG; // this thread belongs to a whole split-group
     const float4 *po = reinterpret_cast<const float4 *>(p.part_o + slot0 * D);
     const float m_first = tid < nsp ? load_partial<DEVICE_COHERENT>(p.part_m + slot0 + tid) : floor_m;
     const float l_first = tid < nsp ? load_partial<DEVICE_COHERENT>(p.part_l + slot0 + tid) : 0.f;
@@ -270,7 +272,7 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
     for (int k = 0; k < 4; ++k)
 #pragma unroll
         for (int v = 0; v < VPT; ++v)
-            x_first[k][v] = sg + k * SG < nsp ? load_partial4<DEVICE_COHERENT>(po + (size_t)(sg + k * SG) * (D / 4) + v * TPG + t)
+            x_first[k][v] = in_group && sg + k * SG < nsp ? load_partial4<DEVICE_COHERENT>(po + (size_t)(sg + k * SG) * (D / 4) + v * TPG + t)
                                               : make_float4(0.f, 0.f, 0.f, 0.f);
 
     float mx = floor_m;
@@ -318,8 +320,8 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
     };
 #pragma unroll
     for (int k = 0; k < 4; ++k)
-        if (sg + k * SG < nsp) add_row(x_first[k], sh.w[sg + k * SG]);
-    int s = sg + 4 * SG;
+        if (in_group && sg + k * SG < nsp) add_row(x_first[k], sh.w[sg + k * SG]);
+    int s = in_group ? sg + 4 * SG : nsp;
     for (; s + 3 * SG < nsp; s += 4 * SG) { // four independent partial rows in flight
         float4 x[4][VPT];
 #pragma unroll
@@ -335,8 +337,10 @@ __device__ __forceinline__ void combine_partials(const Params &p, int bh, int ns
         for (int v = 0; v < VPT; ++v) x[v] = load_partial4<DEVICE_COHERENT>(po + (size_t)s * (D / 4) + v * TPG + t);
         add_row(x, sh.w[s]);
     }
+    if (in_group) {
 #pragma unroll
-    for (int v = 0; v < VPT; ++v) sh.acc[sg][v * TPG + t] = acc[v];
+        for (int v = 0; v < VPT; ++v) sh.acc[sg][v * TPG + t] = acc[v];
+    }
     __syncthreads();
     for (int d4 = tid; d4 < D / 4; d4 += kCombineThreads) {
         float4 r = sh.acc[0][d4];
@@ -374,6 +378,14 @@ __global__ __launch_bounds__(kCombineThreads) void decode_attn_combine_kernel(co
 
 // ---------------------------------------------------------------- streaming (split) kernel
 
+// Lanes that share one cache row of `chunks` 16-byte chunks: the next power of two, at most a wave.
+constexpr int lanes_per_row(int chunks)
+{
+    int n = 1;
+    while (n < chunks && n < 64) n *= 2;
+    return n;
+}
+
 #ifndef FLATTN_MIN_WAVES_PER_EU
 #define FLATTN_MIN_WAVES_PER_EU 8
 #endif
@@ -384,7 +396,9 @@ template <typename T, int D>
 constexpr int min_waves_per_eu()
 {
     constexpr int cpl = (D / Vec16<T>::N) <= 64 ? 1 : (D / Vec16<T>::N) / 64;
-    if (D * (int)sizeof(T) < 128) return 4; // 16 rows per wave: the group merge needs the registers
+    if (lanes_per_row(D / Vec16<T>::N) != D / Vec16<T>::N && cpl == 1) return 4; // padded lane groups (96): the extra
+                                                                                  // predicate spills at 64 registers
+    if (lanes_per_row(D / Vec16<T>::N) < 8) return 4; // 16 rows per wave: the group merge needs the registers
     return cpl == 1 ? FLATTN_MIN_WAVES_PER_EU : (cpl == 2 ? 4 : 2);
 }
 
@@ -400,13 +414,15 @@ void decode_attn_split_kernel(const Params p)
     typedef typename Vec16<T>::type V;
     constexpr int VEC = Vec16<T>::N;
     constexpr int CH = D / VEC;             // 16-byte chunks per row
-    constexpr int LPR = CH < 64 ? CH : 64;  // lanes per row
-    constexpr int CPL = CH / LPR;           // chunks per lane
+    constexpr int LPR = lanes_per_row(CH);  // lanes per row: a power of two, for the butterfly reductions
+    constexpr int CPL = (CH + LPR - 1) / LPR; // chunks per lane
+    constexpr bool PADDED = LPR * CPL != CH; // size_per_head 96: the last lanes of a row's group own no chunk; they load
+                                             // out of range (zeros) and add zeros to every sum
     constexpr int GPW = 64 / LPR;           // rows per wave per load instruction
     constexpr int GROUPS = WAVES * GPW;     // rows per workgroup per load instruction
     constexpr int EPL = CPL * VEC;          // elements of a row owned by one lane
     constexpr int ROW_BYTES = D * (int)sizeof(T);
-    static_assert(CH * VEC == D && LPR * CPL == CH, "head size must tile into 16-byte chunks");
+    static_assert(CH * VEC == D && (!PADDED || CPL == 1), "head size must tile into 16-byte chunks");
 
     __shared__ float s_o[GROUPS][D];
     __shared__ float s_m[GROUPS];
@@ -444,7 +460,8 @@ void decode_attn_split_kernel(const Params p)
     // "scalar base + vector offset" with no per-row 64-bit vector address arithmetic.
     const char *Kb = reinterpret_cast<const char *>(p.k_cache) + (size_t)bh * L * ROW_BYTES;
     const char *Vb = reinterpret_cast<const char *>(p.v_cache) + (size_t)bh * L * ROW_BYTES;
-    const uint32_t lane_off = (uint32_t)(group * ROW_BYTES + lig * 16);
+    const bool has_chunk = !PADDED || lig < CH;
+    const uint32_t lane_off = has_chunk ? (uint32_t)(group * ROW_BYTES + lig * 16) : kLaneOutOfRange;
     const float *mrow = HAS_MASK ? p.attn_mask + (size_t)P * p.mask_ld : nullptr;
     // descriptors of this (b,h)'s K rows, V rows and mask row; row offsets go into the scalar offset
     // (the host checks that L * ROW_BYTES fits 32 bits)
@@ -506,6 +523,11 @@ void decode_attn_split_kernel(const Params p)
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
         const int e0 = (c * LPR + lig) * VEC;
+        if (PADDED && !has_chunk) {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) qr[c * VEC + i] = 0.f;
+            continue;
+        }
         float x[VEC];
         load_token_chunk<T, VEC>(p.q, (size_t)bh * D + e0, is_i32, inp_scale,
                                  is_i32 ? p.wq_scale + h * D + e0 : nullptr, x);
@@ -597,6 +619,11 @@ void decode_attn_split_kernel(const Params p)
 #pragma unroll
         for (int c = 0; c < CPL; ++c) {
             const int e0 = (c * LPR + lig) * VEC;
+            if (PADDED && !has_chunk) { // no chunk of the row: nothing to load or store, zeros into the sums
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) kf[c * VEC + i] = vf[c * VEC + i] = 0.f;
+                continue;
+            }
             float kx[VEC], vx[VEC];
             load_token_chunk<T, VEC>(p.k_new, (size_t)bh * D + e0, is_i32, inp_scale,
                                      is_i32 ? p.wk_scale + h * D + e0 : nullptr, kx);
@@ -642,6 +669,7 @@ void decode_attn_split_kernel(const Params p)
 #pragma unroll
     for (int c = 0; c < CPL; ++c) {
         const int e0 = (c * LPR + lig) * VEC;
+        if (PADDED && !has_chunk) continue;
 #pragma unroll
         for (int i = 0; i < VEC; i += 4)
             *reinterpret_cast<float4 *>(&s_o[group][e0 + i]) =
@@ -678,9 +706,21 @@ void decode_attn_split_kernel(const Params p)
 
     if constexpr (FUSED) {
         if (!p.direct) {
-            // The partial went out through device-coherent stores; the barrier waits until every store of
-            // the workgroup has been performed.  Then the workgroup counts itself in, and the last one
-            // to arrive for this (b,h) merges: its device-coherent loads see every partial counted before.
+            // Ordering of publish -> count -> merge, step by step:
+            //  1. the partial went out through device-coherent stores (sc1: written through to memory that
+            //     every XCD sees);
+            //  2. every thread waits until the memory system has acknowledged ITS stores (vmcnt counts
+            //     stores on this architecture).  A workgroup barrier alone does not: it orders at workgroup
+            //     scope only, and the counter below lives in another channel than the partials;
+            //  3. the barrier: every thread of the workgroup has passed step 2, so all of the workgroup's
+            //     partial is in memory.  Steps 2 + 3 are the release;
+            //  4. one thread counts the workgroup in with a device-scope read-modify-write, executed at
+            //     the memory side, and waits for the returned value before it writes s_last;
+            //  5. the barrier, after which the last workgroup to arrive knows it is the last: every other
+            //     workgroup of this (b,h) incremented before it, hence finished steps 1-3 before;
+            //  6. its device-coherent (sc1) loads are issued after step 5 and bypass the caches that could
+            //     hold stale lines.  Steps 4-6 are the acquire.
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
             const int nsp = active_splits(p, P);
             if (tid == 0) {

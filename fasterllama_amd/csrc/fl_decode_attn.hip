@@ -5,7 +5,9 @@
 
 #include <atomic>
 #include <cmath>
+#include <cstddef>
 #include <cstdint>
+#include <cstring>
 #include <type_traits>
 
 #include "../../include/fl_decode_attn.h"
@@ -55,21 +57,40 @@ int device_cus()
 
 bool head_dim_ok(int D)
 {
-    return D == 32 || D == 64 || D == 128 || D == 256 || D == 512 || D == 1024;
+    // the reference's set: the multiples of 32 up to 128 (decoder_kernels.cu:564-571, :640, :960) and 256, 512, 1024
+    return D == 32 || D == 64 || D == 96 || D == 128 || D == 256 || D == 512 || D == 1024;
+}
+
+// The caller's struct, struct_size bytes of it, copied into a zeroed struct of this build: members the caller's
+// header did not have yet read as zero / NULL.  MIN is the size of the first layout that carried struct_size.
+constexpr size_t kDescMinBytes = offsetof(fl_attn_desc, flags) + sizeof(int32_t);
+constexpr size_t kIoMinBytes = offsetof(fl_attn_io, mask_tile_classes) + sizeof(void *);
+
+template <typename S>
+int import_struct(const S *in, S *out, size_t min_bytes)
+{
+    if (!in) return FL_ATTN_ERR_NULL_POINTER;
+    uint32_t n;
+    std::memcpy(&n, in, sizeof n); // struct_size is the first member of both structs
+    if (n < min_bytes || n > sizeof(S)) return FL_ATTN_ERR_STRUCT_SIZE;
+    std::memset(static_cast<void *>(out), 0, sizeof(S));
+    std::memcpy(static_cast<void *>(out), in, n);
+    return FL_ATTN_OK;
 }
 
 int validate_desc(const fl_attn_desc *d)
 {
-    if (!d) return FL_ATTN_ERR_NULL_POINTER;
     if (d->dtype != FL_ATTN_F32 && d->dtype != FL_ATTN_F16) return FL_ATTN_ERR_DTYPE;
     if (d->batch_size <= 0 || d->head_num <= 0 || d->total_len <= 0) return FL_ATTN_ERR_SHAPE;
     if (d->batch_size > 65535 || d->head_num > 65535) return FL_ATTN_ERR_SHAPE;
     if (!head_dim_ok(d->size_per_head)) return FL_ATTN_ERR_HEAD_DIM;
     if (d->nsplit < 0 || d->nsplit > kMaxSplits || (d->flags & ~FL_ATTN_FLAG_FAST_PROMPT_QK) != 0) return FL_ATTN_ERR_ARGUMENT;
     if (!(d->softmax_scale >= 0.f) || std::isinf(d->softmax_scale)) return FL_ATTN_ERR_ARGUMENT;
-    // row offsets inside one (b,h) slice of a cache are 32-bit byte offsets in the kernels; the prompt-phase kernels
-    // form them for whole 32-row tiles, up to 63 rows past the last one (those rows fail the range check and read as zeros)
-    if (((int64_t)d->total_len + 64) * d->size_per_head * (d->dtype == FL_ATTN_F16 ? 2 : 4) > (int64_t)UINT32_MAX) return FL_ATTN_ERR_SHAPE;
+    // Row offsets inside one (b,h) slice of a cache are 32-bit byte offsets in the kernels, and the buffer descriptors
+    // of the streaming kernel span 2^31 bytes from the slice's base: a slice stays below that, with room for the whole
+    // tiles the prompt-phase kernels address past the last row (up to 63 rows, which fail the range check and read as
+    // zeros).
+    if (((int64_t)d->total_len + 64) * d->size_per_head * (d->dtype == FL_ATTN_F16 ? 2 : 4) >= ((int64_t)1 << 31)) return FL_ATTN_ERR_SHAPE;
     // the streaming grid is one-dimensional: B*H*splits workgroups must fit the 2^31 limit
     if ((int64_t)d->batch_size * d->head_num > (int64_t)INT32_MAX / kMaxSplits) return FL_ATTN_ERR_SHAPE;
     return FL_ATTN_OK;
@@ -79,8 +100,7 @@ int validate_desc(const fl_attn_desc *d)
 int rows_per_tile(const fl_attn_desc *d, int unroll)
 {
     const int vec = d->dtype == FL_ATTN_F16 ? 8 : 4;
-    const int ch = d->size_per_head / vec;
-    const int lpr = ch < 64 ? ch : 64;
+    const int lpr = flattn::lanes_per_row(d->size_per_head / vec);
     return kWaves * (64 / lpr) * unroll;
 }
 
@@ -169,6 +189,15 @@ void make_plan(const fl_attn_desc *d, int ctx, bool ragged, fl_attn_plan *plan)
     plan->two_pass = plan->nsplit <= 1 ? 0 : (fused_merge_pays(d, plan->nsplit) ? 2 : 1);
 }
 
+// Every entry point works on its own copy of the caller's descriptor (see import_struct).
+int import_desc(const fl_attn_desc **desc, fl_attn_desc *copy)
+{
+    const int st = import_struct(*desc, copy, kDescMinBytes);
+    if (st != FL_ATTN_OK) return st;
+    *desc = copy;
+    return validate_desc(copy);
+}
+
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 // Row stride of the persistent mask tile class table: the 32-row blocks of one key tile, padded to whole words.
@@ -214,9 +243,24 @@ size_t workspace_need(const fl_attn_desc *d) { return workspace_layout(d).total;
 
 // Scratch memory of fl_decode_attn_forward_noalloc: one array per GPU, part of the library's code
 // object, so that entry point never allocates.  Static storage starts out zero, which is the state the
-// arrival counters need, and every launch that uses them leaves them zero again.
+// arrival counters need, and every launch that uses them leaves them zero again.  The counters own the
+// last kScratchCounterBytes of the array, whatever the shape of the call: the float output and the split
+// partials of any call stay below them, so no call can leave a non-zero word where a later call with
+// another batch or head count expects a counter.
 constexpr size_t kScratchBytes = FL_ATTN_NOALLOC_SCRATCH_BYTES;
+constexpr size_t kScratchCounterBytes = 64u << 10; // 16384 (batch, head) pairs; larger steps merge in a second launch
+constexpr size_t kScratchDataBytes = kScratchBytes - kScratchCounterBytes;
 static __device__ __align__(256) unsigned char g_scratch[kScratchBytes];
+
+// Layout of a step inside the library's own array: data sections packed from byte 0, counters in their fixed tail.
+WorkspaceLayout scratch_layout(const fl_attn_desc *d, int cap)
+{
+    WorkspaceLayout w = workspace_layout(d, cap);
+    const size_t shift = w.tmp_out; // the caller-workspace layout starts with its counters
+    w.tmp_out -= shift; w.part_o -= shift; w.part_m -= shift; w.part_l -= shift; w.total -= shift;
+    w.arrivals = kScratchDataBytes;
+    return w;
+}
 
 // Device address of g_scratch on the current device (each GPU holds its own copy at its own address);
 // looked up once per device.  In host code the array's name is only a handle for this lookup.
@@ -256,6 +300,7 @@ hipError_t dispatch_combine(int D, const Params &p, int bh, hipStream_t stream)
     switch (D) {
     case 32: return launch_combine<32>(p, bh, stream);
     case 64: return launch_combine<64>(p, bh, stream);
+    case 96: return launch_combine<96>(p, bh, stream);
     case 128: return launch_combine<128>(p, bh, stream);
     case 256: return launch_combine<256>(p, bh, stream);
     case 512: return launch_combine<512>(p, bh, stream);
@@ -296,6 +341,7 @@ hipError_t dispatch_split(int D, const Params &p, dim3 grid, hipStream_t stream)
     switch (D) {
     case 32: return launch_split<T, 32>(p, grid, stream);
     case 64: return launch_split<T, 64>(p, grid, stream);
+    case 96: return launch_split<T, 96>(p, grid, stream);
     case 128: return launch_split<T, 128>(p, grid, stream);
     case 256: return launch_split<T, 256>(p, grid, stream);
     case 512: return launch_split<T, 512>(p, grid, stream);
@@ -332,7 +378,7 @@ template <typename T, int D>
 hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
 {
     constexpr int VEC = flattn::Vec16<T>::N;
-    constexpr int LPR = D / VEC < 64 ? D / VEC : 64;
+    constexpr int LPR = flattn::lanes_per_row(D / VEC);
     constexpr int ROWS = 256 / LPR;
     // lane groups of the append kernel: one per token and four heads for fp16 inputs where the head count allows
     // (B=8,S=1024: 49.0 -> 44.2 us; FP32 rows and int32 accumulators, twice the bytes per lane already, gain
@@ -374,6 +420,7 @@ hipError_t dispatch_prefill(int D, const flattn::PrefillParams &p, hipStream_t s
     switch (D) {
     case 32: return launch_prefill<T, 32>(p, stream);
     case 64: return launch_prefill<T, 64>(p, stream);
+    case 96: return launch_prefill<T, 96>(p, stream);
     case 128: return launch_prefill<T, 128>(p, stream);
     case 256: return launch_prefill<T, 256>(p, stream);
     case 512: return launch_prefill<T, 512>(p, stream);
@@ -388,7 +435,7 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 extern "C" {
 
-int fl_attn_version(void) { return 200; }
+int fl_attn_version(void) { return 300; }
 
 int fl_attn_last_hip_error(void) { return g_last_hip_error; }
 
@@ -398,7 +445,7 @@ const char *fl_attn_strerror(int status)
     case FL_ATTN_OK: return "ok";
     case FL_ATTN_ERR_NULL_POINTER: return "a required pointer is NULL";
     case FL_ATTN_ERR_HEAD_DIM:
-        return "invalid size_per_head (32, 64, 128, 256, 512 or 1024)";
+        return "invalid size_per_head (32, 64, 96, 128, 256, 512 or 1024)";
     case FL_ATTN_ERR_SHAPE: return "invalid batch_size / head_num / total_len";
     case FL_ATTN_ERR_POSITION: return "start_pos or rope_row out of range for total_len";
     case FL_ATTN_ERR_WORKSPACE: return "workspace missing, too small or not 256-byte aligned";
@@ -406,6 +453,8 @@ const char *fl_attn_strerror(int status)
     case FL_ATTN_ERR_HIP: return "a HIP runtime call failed";
     case FL_ATTN_ERR_ALIGNMENT: return "tensor base pointers must be 16-byte aligned";
     case FL_ATTN_ERR_ARGUMENT: return "inconsistent arguments";
+    case FL_ATTN_ERR_STRUCT_SIZE:
+        return "struct_size of fl_attn_desc / fl_attn_io is not set or comes from a newer header than this library";
     case FL_ATTN_ERR_SCRATCH_LIMIT:
         return "the step needs more scratch than fl_decode_attn_forward_noalloc holds (FL_ATTN_NOALLOC_SCRATCH_BYTES); "
                "use fl_decode_attn_forward with a caller-owned workspace";
@@ -416,7 +465,8 @@ const char *fl_attn_strerror(int status)
 int fl_decode_attn_workspace_bytes(const fl_attn_desc *desc, size_t *bytes)
 {
     if (!bytes) return FL_ATTN_ERR_NULL_POINTER;
-    int st = validate_desc(desc);
+    fl_attn_desc desc_copy;
+    int st = import_desc(&desc, &desc_copy);
     if (st != FL_ATTN_OK) return st;
     *bytes = workspace_need(desc);
     return FL_ATTN_OK;
@@ -425,7 +475,8 @@ int fl_decode_attn_workspace_bytes(const fl_attn_desc *desc, size_t *bytes)
 int fl_kv_cache_bytes(const fl_attn_desc *desc, size_t *bytes)
 {
     if (!bytes) return FL_ATTN_ERR_NULL_POINTER;
-    int st = validate_desc(desc);
+    fl_attn_desc desc_copy;
+    int st = import_desc(&desc, &desc_copy);
     if (st != FL_ATTN_OK) return st;
     const size_t e = desc->dtype == FL_ATTN_F16 ? 2 : 4;
     *bytes = (size_t)desc->batch_size * desc->head_num * (size_t)desc->total_len * desc->size_per_head * e;
@@ -435,7 +486,8 @@ int fl_kv_cache_bytes(const fl_attn_desc *desc, size_t *bytes)
 int fl_decode_attn_plan(const fl_attn_desc *desc, int32_t ctx, int32_t ragged, fl_attn_plan *plan)
 {
     if (!plan) return FL_ATTN_ERR_NULL_POINTER;
-    int st = validate_desc(desc);
+    fl_attn_desc desc_copy;
+    int st = import_desc(&desc, &desc_copy);
     if (st != FL_ATTN_OK) return st;
     if (ctx < 1 || ctx > desc->total_len) return FL_ATTN_ERR_POSITION;
     make_plan(desc, ctx, ragged != 0, plan);
@@ -448,11 +500,15 @@ namespace {
 
 // The decode step behind every entry point.  own_scratch: take the split partials and arrival
 // counters from the library's per-GPU scratch array instead of io->workspace (no allocation either way).
-int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_stream, int passes, bool own_scratch)
+int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io_in, void *hip_stream, int passes, bool own_scratch)
 {
-    int st = validate_desc(desc);
+    fl_attn_desc desc_copy;
+    int st = import_desc(&desc, &desc_copy);
     if (st != FL_ATTN_OK) return st;
-    if (!io) return FL_ATTN_ERR_NULL_POINTER;
+    fl_attn_io io_copy;
+    st = import_struct(io_in, &io_copy, kIoMinBytes);
+    if (st != FL_ATTN_OK) return st;
+    const fl_attn_io *io = &io_copy;
     if ((passes & ~3) != 0 || passes == 0) return FL_ATTN_ERR_ARGUMENT;
     if (!io->q || !io->k_new || !io->v_new || !io->k_cache || !io->v_cache || !io->freq_cis)
         return FL_ATTN_ERR_NULL_POINTER;
@@ -492,12 +548,12 @@ int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_str
 
     const bool direct = plan.nsplit == 1; // the streaming kernel normalises and writes the output itself
     const bool need_ws = !direct || (quant && !io->out);
-    const WorkspaceLayout wl = workspace_layout(desc, cap);
+    const WorkspaceLayout wl = own_scratch ? scratch_layout(desc, cap) : workspace_layout(desc, cap);
     char *ws = static_cast<char *>(io->workspace);
     if (own_scratch) {
         ws = nullptr;
         if (need_ws) {
-            if (wl.total > kScratchBytes) return FL_ATTN_ERR_SCRATCH_LIMIT;
+            if (wl.total > kScratchDataBytes) return FL_ATTN_ERR_SCRATCH_LIMIT;
             if (!check_hip(scratch_address(&ws))) return FL_ATTN_ERR_HIP;
         }
     } else if (need_ws) {
@@ -506,7 +562,9 @@ int decode_forward(const fl_attn_desc *desc, const fl_attn_io *io, void *hip_str
     }
     // One launch with the merge inside needs arrival counters that are zero: the library's own scratch
     // always is (between launches), the caller's workspace when it says so.
-    const bool fused = plan.two_pass == 2 && passes == 3 && (own_scratch || (io->flags & FL_ATTN_IO_WORKSPACE_READY) != 0);
+    const bool counters_fit = (size_t)desc->batch_size * desc->head_num * sizeof(int32_t) <= kScratchCounterBytes;
+    const bool fused = plan.two_pass == 2 && passes == 3 &&
+                       (own_scratch ? counters_fit : (io->flags & FL_ATTN_IO_WORKSPACE_READY) != 0);
 
     const int D = desc->size_per_head;
     Params p{};
@@ -569,7 +627,8 @@ int fl_decode_attn_forward_noalloc(const fl_attn_desc *desc, const fl_attn_io *i
 
 int fl_decode_attn_workspace_init(const fl_attn_desc *desc, void *workspace, size_t workspace_bytes, void *hip_stream)
 {
-    int st = validate_desc(desc);
+    fl_attn_desc desc_copy;
+    int st = import_desc(&desc, &desc_copy);
     if (st != FL_ATTN_OK) return st;
     const WorkspaceLayout wl = workspace_layout(desc);
     if (!workspace || workspace_bytes < wl.total || (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
@@ -587,7 +646,8 @@ int fl_decode_attn_workspace_init(const fl_attn_desc *desc, void *workspace, siz
 int fl_prefill_attn_workspace_bytes(const fl_attn_desc *desc, int32_t seq_len, size_t *bytes)
 {
     if (!bytes) return FL_ATTN_ERR_NULL_POINTER;
-    int st = validate_desc(desc);
+    fl_attn_desc desc_copy;
+    int st = import_desc(&desc, &desc_copy);
     if (st != FL_ATTN_OK) return st;
     if (!prefill_head_dim_ok(desc->size_per_head)) return FL_ATTN_ERR_HEAD_DIM;
     if (seq_len < 1 || seq_len > desc->total_len) return FL_ATTN_ERR_POSITION;
@@ -595,12 +655,16 @@ int fl_prefill_attn_workspace_bytes(const fl_attn_desc *desc, int32_t seq_len, s
     return FL_ATTN_OK;
 }
 
-int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int32_t seq_len, void *hip_stream)
+int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io_in, int32_t seq_len, void *hip_stream)
 {
-    int st = validate_desc(desc);
+    fl_attn_desc desc_copy;
+    int st = import_desc(&desc, &desc_copy);
     if (st != FL_ATTN_OK) return st;
     if (!prefill_head_dim_ok(desc->size_per_head)) return FL_ATTN_ERR_HEAD_DIM;
-    if (!io) return FL_ATTN_ERR_NULL_POINTER;
+    fl_attn_io io_copy;
+    st = import_struct(io_in, &io_copy, kIoMinBytes);
+    if (st != FL_ATTN_OK) return st;
+    const fl_attn_io *io = &io_copy;
     if (!io->q || !io->k_new || !io->v_new || !io->k_cache || !io->v_cache || !io->freq_cis)
         return FL_ATTN_ERR_NULL_POINTER;
     const bool quant = io->out_int8 != nullptr;
@@ -661,7 +725,8 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
 int fl_prefill_mask_classes_bytes(const fl_attn_desc *desc, size_t *bytes)
 {
     if (!bytes) return FL_ATTN_ERR_NULL_POINTER;
-    int st = validate_desc(desc);
+    fl_attn_desc desc_copy;
+    int st = import_desc(&desc, &desc_copy);
     if (st != FL_ATTN_OK) return st;
     const size_t n = ((size_t)desc->total_len + 31) / 32;
     *bytes = n * class_table_ld(desc->total_len);
@@ -671,7 +736,8 @@ int fl_prefill_mask_classes_bytes(const fl_attn_desc *desc, size_t *bytes)
 int fl_prefill_mask_classify(const fl_attn_desc *desc, const float *attn_mask, int64_t mask_ld, void *classes,
                              size_t classes_bytes, void *hip_stream)
 {
-    int st = validate_desc(desc);
+    fl_attn_desc desc_copy;
+    int st = import_desc(&desc, &desc_copy);
     if (st != FL_ATTN_OK) return st;
     if (!attn_mask || !classes) return FL_ATTN_ERR_NULL_POINTER;
     const int L = desc->total_len;

@@ -24,6 +24,7 @@ namespace FasterLLaMA
         fl_attn_desc makeDesc(int B, int H, int D, int L, int nsplit)
         {
             fl_attn_desc d{};
+            d.struct_size = sizeof d;
             d.batch_size = B;
             d.head_num = H;
             d.size_per_head = D;
@@ -98,12 +99,23 @@ namespace FasterLLaMA
         return (int)n;
     }
 
+    // The reference's initialize() is pointer carving and nothing else (open_decoder.cu:25-51), and its driver
+    // calls it before every layer of every step with the same buf (decoding_sampling.cu:232-258).  Same here:
+    // a call with the workspace that is already prepared only copies `param`.  The one-time work — sizing the
+    // scratch areas and a small kernel that zeroes the arrival counters of the decode scratch — happens on the
+    // first call, and again only when `buf` changes.  The tile classes of the mask stay valid as long as
+    // param.attn_mask is the pointer they were computed from (contents that change behind the same pointer are
+    // the caller's classifyMask() call).
     template <OperationType OpType_, OperationType QuantizationType>
     void OpenDecoder<OpType_, QuantizationType>::initialize(DecoderInitParam<DataType_, weight_DataType_> param, char *buf)
     {
-        param_ = param;
         if (!buf)
             throw std::runtime_error("[FL][ERROR] initialize: workspace is null");
+        param_ = param;
+        if (mask_classified_ && param_.attn_mask != classified_mask_)
+            mask_classified_ = false;
+        if (buf == prepared_buf_)
+            return;
         const size_t tokens = (size_t)batch_size_ * (size_t)(max_prompt_len_ > 1 ? max_prompt_len_ : 1);
         char *p = reinterpret_cast<char *>(roundUp(reinterpret_cast<uintptr_t>(buf), 256));
         from_tensor_int8_buf_ = reinterpret_cast<int8_t *>(p);
@@ -124,12 +136,13 @@ namespace FasterLLaMA
         prompt_workspace_bytes_ = promptWorkspaceBytes();
         p += roundUp(prompt_workspace_bytes_, 256);
         mask_classes_ = p;
-        mask_classified_ = false;
+        mask_classified_ = false; // another table address: nothing has been written there
         // arrival counters of the decode scratch start at zero (a small kernel on the caller's stream); from
         // here on a decode step whose context is split is a single launch
         fl_attn_desc d = makeDesc<float>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
         throwOnStatus(fl_decode_attn_workspace_init(&d, attn_workspace_, attn_workspace_bytes_, param_.stream), "initialize");
         throwOnStatus(fl_prefill_mask_classes_bytes(&d, &mask_classes_bytes_), "initialize");
+        prepared_buf_ = buf;
     }
 
     template <OperationType OpType_, OperationType QuantizationType>
@@ -143,6 +156,7 @@ namespace FasterLLaMA
         throwOnStatus(fl_prefill_mask_classify(&d, param_.attn_mask, total_len_, mask_classes_, mask_classes_bytes_, param_.stream),
                       "classifyMask");
         mask_classified_ = true;
+        classified_mask_ = param_.attn_mask;
     }
 
     template <OperationType OpType_, OperationType QuantizationType>
@@ -156,6 +170,7 @@ namespace FasterLLaMA
             throw std::runtime_error("[FL][ERROR] forward: initialize() has not been called");
         fl_attn_desc desc = makeDesc<CacheT>(batch_size_, head_num_, size_per_head_, total_len_, nsplit_);
         fl_attn_io io{};
+        io.struct_size = sizeof io;
         io.q = q;
         io.k_new = k;
         io.v_new = v;

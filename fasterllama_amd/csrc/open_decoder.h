@@ -147,6 +147,8 @@ namespace FasterLLaMA
         char *mask_classes_ = nullptr;            // tile classes of param_.attn_mask, see classifyMask()
         size_t mask_classes_bytes_ = 0;
         bool mask_classified_ = false;
+        const float *classified_mask_ = nullptr;  // the attn_mask pointer the table was computed from
+        const char *prepared_buf_ = nullptr;      // the workspace whose arrival counters initialize() has zeroed
 
         size_t decodeWorkspaceBytes() const;
         size_t promptWorkspaceBytes() const;
@@ -181,7 +183,11 @@ namespace FasterLLaMA
         // ---- additions -------------------------------------------------------------------------
         void setExternalStages(const DecoderExternalStages<DataType_> &stages) { stages_ = stages; }
         void setLiteralRopeRow(bool literal) { literal_rope_row_ = literal; }
-        void setContextSplits(int nsplit) { nsplit_ = nsplit; } // 0 = chosen by the library
+        void setContextSplits(int nsplit) // 0 = chosen by the library; the scratch areas are sized anew by the next initialize()
+        {
+            if (nsplit != nsplit_) prepared_buf_ = nullptr;
+            nsplit_ = nsplit;
+        }
         // Classifies the tiles of param_.attn_mask once (on param_.stream), so that prompt-phase calls do not
         // classify the rows they use on every call.  Call it after the mask has been filled, and again when its
         // contents change; without it every prompt-phase call classifies for itself.

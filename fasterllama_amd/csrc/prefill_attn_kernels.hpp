@@ -53,8 +53,8 @@ __global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillP
     typedef typename Vec16<T>::type V;
     constexpr int VEC = Vec16<T>::N;
     constexpr int CH = D / VEC;
-    constexpr int LPR = CH < 64 ? CH : 64;
-    constexpr int CPL = CH / LPR;
+    constexpr int LPR = lanes_per_row(CH); // a power of two; at size_per_head 96 the last lanes of a group own no chunk
+    constexpr int CPL = (CH + LPR - 1) / LPR;
     constexpr int ROWS = 256 / LPR;
 
     const int HG = p.H / HPT; // head groups per token (the launcher picks HPT so that it divides H)
@@ -62,6 +62,7 @@ __global__ __launch_bounds__(256) void prefill_rope_append_kernel(const PrefillP
     const int64_t g = (int64_t)blockIdx.x * ROWS + threadIdx.x / LPR; // index into [B,S,H/HPT]
     if (g >= groups) return;
     const int lig = threadIdx.x % LPR;
+    if (LPR * CPL != CH && lig >= CH) return;
     const int h0 = (int)(g % HG) * HPT;
     const int64_t bs = g / HG;
     const int s = (int)(bs % p.S), b = (int)(bs / p.S);
@@ -309,7 +310,7 @@ void prefill_attn_kernel(const PrefillParams p)
     constexpr int NC = D / 8;
     constexpr int NDT = D / 32;
     constexpr int CPR = D / VEC; // 16-byte chunks per cache row
-    static_assert(D % 32 == 0, "head size must be a multiple of 32");
+    static_assert(D % 32 == 0, "head size must be a multiple of 32"); // NC = D / 8 is even: the score chunks go in pairs
     static_assert(std::is_same<T, float>::value, "the FP32-MFMA kernel works on FP32 caches");
 
     // D >= 64: the key tiles go from global memory straight into LDS, two buffers deep, so the next tile
@@ -320,9 +321,9 @@ void prefill_attn_kernel(const PrefillParams p)
     // (the 16 lanes of a 128-bit read pass, keys r..r+15 at one d, hit 16 different bank groups), V keeps it at
     // c ^ 8 for the rows with bit 2 set (the two key rows of a 32-bit read, four apart, use different halves
     // of the banks).  Each lane applies the swizzle to the GLOBAL address it loads from.
-    constexpr bool DMA = D >= 64;
+    constexpr bool DMA = D == 64 || D == 128; // (96: rows of 384 bytes do not tile the 1 KB of a direct load; staged path)
     constexpr int ROWB = D * 4;          // bytes per cache row
-    constexpr int RPI = 1024 / ROWB;     // rows per direct load
+    constexpr int RPI = DMA ? 1024 / ROWB : 1; // rows per direct load
     constexpr int NI = DMA ? BN / RPI / 4 : 1; // direct loads per wave, tile and matrix
     constexpr uint32_t TILEB = BN * ROWB; // bytes of one K (or V) tile
     constexpr int LDK = D + 4;           // staged path: padded LDS row (floats), rows start 4 banks apart
@@ -405,19 +406,30 @@ void prefill_attn_kernel(const PrefillParams p)
         constexpr bool DIRECT = decltype(direct_tag)::value;
         const char *kt = reinterpret_cast<const char *>(smem) + (DIRECT ? (uint32_t)buf * 2u * TILEB : 0u);
         const char *vt = kt + TILEB;
-        // S^T tile: 32 keys x 32 queries, contraction over D
-        floatx16 st;
+        // S^T tile: 32 keys x 32 queries, contraction over D.  Two accumulators, even and odd chunks, added at the
+        // end: each sums D/2 products, so the partial sums stay smaller and the rounding error of a score is
+        // about 0.7 of what one sequential chain over D leaves (the scores' error is a relative error of the weights).
+        floatx16 st, st1;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) st[v] = 0.f;
+        for (int v = 0; v < 16; ++v) st[v] = st1[v] = 0.f;
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
+        for (int c = 0; c < NC; c += 2) {
             const float4 ka = DIRECT ? *reinterpret_cast<const float4 *>(kt + (k_swz ^ (uint32_t)(c << 5)))
                                      : *reinterpret_cast<const float4 *>(&sK[qi][8 * c + 4 * hf]);
+            const float4 kb = DIRECT ? *reinterpret_cast<const float4 *>(kt + (k_swz ^ (uint32_t)((c + 1) << 5)))
+                                     : *reinterpret_cast<const float4 *>(&sK[qi][8 * (c + 1) + 4 * hf]);
             st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.x, qreg[c][0], st, 0, 0, 0);
+            st1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kb.x, qreg[c + 1][0], st1, 0, 0, 0);
             st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.y, qreg[c][1], st, 0, 0, 0);
+            st1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kb.y, qreg[c + 1][1], st1, 0, 0, 0);
             st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.z, qreg[c][2], st, 0, 0, 0);
+            st1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kb.z, qreg[c + 1][2], st1, 0, 0, 0);
             st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.w, qreg[c][3], st, 0, 0, 0);
+            st1 = __builtin_amdgcn_mfma_f32_32x32x2f32(kb.w, qreg[c + 1][3], st1, 0, 0, 0);
         }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) st[v] += st1[v];
+        __builtin_amdgcn_sched_barrier(0);
 
         // softmax update of this lane's query: v = s*scale + mask, floor -1e9 (decoder_kernels.cu:811-820)
         float sc[16];
@@ -445,16 +457,25 @@ void prefill_attn_kernel(const PrefillParams p)
         }
 
         // O^T += V^T P^T: contraction over the 32 keys, two per MFMA (key of step t in half hf:
-        // 8*(t/4) + 4*hf + (t%4), the key whose probability this lane holds in sc[t])
+        // 8*(t/4) + 4*hf + (t%4), the key whose probability this lane holds in sc[t]).  The tile's 32 terms are
+        // summed in an accumulator of their own and added to the running output once: the running sums, which
+        // carry the large partial results, are rounded once per tile instead of once per key.
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
+        for (int dt = 0; dt < NDT; ++dt) {
+            floatx16 part;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) part[v] = 0.f;
 #pragma unroll
             for (int t = 0; t < 16; ++t) {
                 const float va = DIRECT ? *reinterpret_cast<const float *>(vt + v_lane + (uint32_t)((((dt & 1) ^ hf) << 7) + (dt >> 1) * 256 +
                                                                                                    (8 * (t / 4) + (t % 4)) * ROWB))
                                         : sV[8 * (t / 4) + 4 * hf + (t % 4)][32 * dt + qi];
-                ot[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(va, sc[t], ot[dt], 0, 0, 0);
+                part = __builtin_amdgcn_mfma_f32_32x32x2f32(va, sc[t], part, 0, 0, 0);
             }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) ot[dt][v] += part[v];
+            __builtin_amdgcn_sched_barrier(0); // one output tile at a time: operands hoisted across tiles cost registers the kernel does not have
+        }
         (void)tc;
     };
     // mask values of this lane's query, gathered straight from global memory: the FP32-MFMA kernel
@@ -711,7 +732,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     constexpr bool DMA = D == 128;
     constexpr int NBUF = DMA ? 3 : 2;       // tile buffers: a direct load is issued two tiles ahead
     constexpr int LDK = DMA ? D : D + 8;    // halfs; padded rows start 4 banks apart (128-bit operand reads)
-    constexpr int LDV = DMA ? D : D + 32;   // halfs; padded rows start 16 banks apart (8 rows x 64 bytes per transposing read)
+    constexpr int LDV = DMA ? D : (D == 96 ? D + 48 : D + 32); // halfs; padded rows start 16 banks apart (8 rows x 64 bytes per transposing read; 8 banks at D = 96)
     constexpr int NC = D / 16;
     constexpr int NDT = D / 32;
     constexpr int CPR = D / 8; // 16-byte chunks per cache row
@@ -857,9 +878,14 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         const int b = bh / p.H, h = bh % p.H;
         const int row0 = p.rope_row < 0 ? P : p.rope_row;
         constexpr int QPL = 32 * CPR / 64;  // 16-byte chunks per lane
-        constexpr int RPI = 64 / CPR;       // query rows per load instruction
-        static_assert(64 % CPR == 0, "a lane keeps its column chunk over all its rows");
-        const int cc = lane % CPR, rl = lane / CPR;
+        // Rows of a power-of-two number of chunks: a lane keeps its column chunk over all its rows (RPI rows per
+        // load instruction).  Otherwise (size_per_head 96: 12 chunks) the wave's 32 * CPR chunks are dealt out
+        // in order, lane + 64 j, and row and column change with j.
+        constexpr bool FIXED_COL = 64 % CPR == 0;
+        constexpr int RPI = FIXED_COL ? 64 / CPR : 1; // query rows per load instruction
+        static_assert((32 * CPR) % 64 == 0, "every lane owns the same number of query chunks");
+        auto q_rl = [&](int j) __attribute__((always_inline)) -> int { return FIXED_COL ? lane / CPR + j * RPI : (lane + 64 * j) / CPR; };
+        auto q_cc = [&](int j) __attribute__((always_inline)) -> int { return FIXED_COL ? lane % CPR : (lane + 64 * j) % CPR; };
         const int q_first = qb * kPrefillQueriesPerBlock + wave * 32;
         _Float16 *const sq = sQ + wave * 32 * LDQ;
         float x[QPL][8];
@@ -869,10 +895,10 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         auto load_queries = [&](auto i32_tag) __attribute__((always_inline)) {
             constexpr bool I32 = decltype(i32_tag)::value != 0;
             constexpr int BATCH = I32 && QPL > 1 ? QPL / 2 : QPL; // int32 accumulators: twice the registers
-            float4 w[2];
-            if constexpr (I32) {
-                w[0] = *reinterpret_cast<const float4 *>(p.wq_scale + h * D + cc * 8);
-                w[1] = *reinterpret_cast<const float4 *>(p.wq_scale + h * D + cc * 8 + 4);
+            float4 w[FIXED_COL ? 1 : BATCH][2];
+            if constexpr (I32 && FIXED_COL) {
+                w[0][0] = *reinterpret_cast<const float4 *>(p.wq_scale + h * D + q_cc(0) * 8);
+                w[0][1] = *reinterpret_cast<const float4 *>(p.wq_scale + h * D + q_cc(0) * 8 + 4);
             }
 #pragma unroll
             for (int j0 = 0; j0 < QPL; j0 += BATCH) {
@@ -882,7 +908,8 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 float4 rf[BATCH][2];
 #pragma unroll
                 for (int jj = 0; jj < BATCH; ++jj) {
-                    const int q = min(q_first + rl + (j0 + jj) * RPI, S - 1);
+                    const int cc = q_cc(j0 + jj);
+                    const int q = min(q_first + q_rl(j0 + jj), S - 1);
                     const int64_t token = (int64_t)b * S + q;
                     const size_t off = (size_t)(token * p.H + h) * D + cc * 8;
                     if constexpr (I32) {
@@ -890,6 +917,10 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                         ri[jj][0] = src[0];
                         ri[jj][1] = src[1];
                         sc[jj] = p.inp_scale[token];
+                        if constexpr (!FIXED_COL) {
+                            w[jj][0] = *reinterpret_cast<const float4 *>(p.wq_scale + h * D + cc * 8);
+                            w[jj][1] = *reinterpret_cast<const float4 *>(p.wq_scale + h * D + cc * 8 + 4);
+                        }
                     } else {
                         rh[jj] = *reinterpret_cast<const half8 *>(reinterpret_cast<const _Float16 *>(p.q) + off);
                     }
@@ -902,8 +933,9 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 for (int jj = 0; jj < BATCH; ++jj) {
                     float v[8];
                     if constexpr (I32) { // decoder_kernels.cu:449-452
+                        const float4 *wj = w[FIXED_COL ? 0 : jj];
                         const int a[8] = {ri[jj][0].x, ri[jj][0].y, ri[jj][0].z, ri[jj][0].w, ri[jj][1].x, ri[jj][1].y, ri[jj][1].z, ri[jj][1].w};
-                        const float ws[8] = {w[0].x, w[0].y, w[0].z, w[0].w, w[1].x, w[1].y, w[1].z, w[1].w};
+                        const float ws[8] = {wj[0].x, wj[0].y, wj[0].z, wj[0].w, wj[1].x, wj[1].y, wj[1].z, wj[1].w};
 #pragma unroll
                         for (int i = 0; i < 8; ++i) v[i] = __fmul_rn(__fmul_rn((float)a[i], sc[jj]), ws[i]);
                     } else {
@@ -928,14 +960,14 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         half8 lo_keep[QSPLIT ? QPL : 1];
 #pragma unroll
         for (int j = 0; j < QPL; ++j) {
-            const bool valid = q_first + rl + j * RPI < S;
+            const bool valid = q_first + q_rl(j) < S;
             half8 hq;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 hq[i] = valid ? (_Float16)x[j][i] : (_Float16)0;
                 if constexpr (QSPLIT) lo_keep[j][i] = valid ? (_Float16)(x[j][i] - (float)hq[i]) : (_Float16)0;
             }
-            *reinterpret_cast<half8 *>(sq + (rl + j * RPI) * LDQ + cc * 8) = hq;
+            *reinterpret_cast<half8 *>(sq + q_rl(j) * LDQ + q_cc(j) * 8) = hq;
         }
         wave_sync();
 #pragma unroll
@@ -943,7 +975,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         if constexpr (QSPLIT) {
             wave_sync();
 #pragma unroll
-            for (int j = 0; j < QPL; ++j) *reinterpret_cast<half8 *>(sq + (rl + j * RPI) * LDQ + cc * 8) = lo_keep[j];
+            for (int j = 0; j < QPL; ++j) *reinterpret_cast<half8 *>(sq + q_rl(j) * LDQ + q_cc(j) * 8) = lo_keep[j];
             wave_sync();
 #pragma unroll
             for (int c = 0; c < NC; ++c) qlo[c] = *reinterpret_cast<const half8 *>(sq + qi * LDQ + 16 * c + 8 * hf);

@@ -47,7 +47,7 @@ extern "C" {
 typedef enum fl_attn_status {
     FL_ATTN_OK = 0,
     FL_ATTN_ERR_NULL_POINTER = -1,  /* a required pointer is NULL */
-    FL_ATTN_ERR_HEAD_DIM = -2,      /* size_per_head not in {32,64,128,256,512,1024}
+    FL_ATTN_ERR_HEAD_DIM = -2,      /* size_per_head not in {32,64,96,128,256,512,1024}
                                        (reference: throw "invalid size_per_head!") */
     FL_ATTN_ERR_SHAPE = -3,         /* non-positive B/H/L, or sizes beyond the grid limits */
     FL_ATTN_ERR_POSITION = -4,      /* start_pos (+1) does not fit in total_len, bad rope_row */
@@ -56,8 +56,10 @@ typedef enum fl_attn_status {
     FL_ATTN_ERR_HIP = -7,           /* a HIP runtime call failed (see fl_attn_last_hip_error) */
     FL_ATTN_ERR_ALIGNMENT = -8,     /* a tensor base is not 16-byte aligned */
     FL_ATTN_ERR_ARGUMENT = -9,      /* inconsistent optional arguments */
-    FL_ATTN_ERR_SCRATCH_LIMIT = -10 /* fl_decode_attn_forward_noalloc: the step needs more scratch than
-                                       FL_ATTN_NOALLOC_SCRATCH_BYTES */
+    FL_ATTN_ERR_SCRATCH_LIMIT = -10, /* fl_decode_attn_forward_noalloc: the step needs more scratch than
+                                        FL_ATTN_NOALLOC_SCRATCH_BYTES */
+    FL_ATTN_ERR_STRUCT_SIZE = -11    /* struct_size of fl_attn_desc / fl_attn_io is not one this library knows:
+                                        not set, or the caller was built against a newer header */
 } fl_attn_status;
 
 enum { FL_ATTN_F32 = 0, FL_ATTN_F16 = 1 };
@@ -82,8 +84,15 @@ enum { FL_ATTN_F32 = 0, FL_ATTN_F16 = 1 };
 /* rope_row value meaning "rotate by the table row of each sequence's own position" */
 #define FL_ATTN_ROPE_AT_POSITION (-1)
 
+/* Both structs start with their own size as the caller's header defines it, so that they can grow at the
+ * end: the library reads struct_size bytes and takes every member beyond them as zero / NULL ("not given").
+ * A size below that of the first layout with this member, or above the library's own, is rejected with
+ * FL_ATTN_ERR_STRUCT_SIZE instead of being read past its end.
+ *   fl_attn_desc d = {sizeof d};  d.batch_size = ...;        fl_attn_io io = {sizeof io};  io.q = ...; */
+
 /* Problem shape; mirrors the OpenDecoder constructor arguments (open_decoder.h:66). */
 typedef struct fl_attn_desc {
+    uint32_t struct_size;  /* sizeof(fl_attn_desc) */
     int32_t batch_size;    /* B */
     int32_t head_num;      /* H */
     int32_t size_per_head; /* D */
@@ -96,6 +105,7 @@ typedef struct fl_attn_desc {
 
 /* Per-call operands; mirrors the arguments of OpenDecoder::forward (open_decoder.h:76-77). */
 typedef struct fl_attn_io {
+    uint32_t struct_size; /* sizeof(fl_attn_io) */
     const void *q;      /* [B,1,H,D] dtype; int32 accumulators when qkv_inp_scale != NULL */
     const void *k_new;  /* same */
     const void *v_new;  /* same */

@@ -22,6 +22,7 @@ static fl_attn_desc desc(int B, int H, int D, int L, int dtype, int nsplit)
 {
     fl_attn_desc d;
     std::memset(&d, 0, sizeof d);
+    d.struct_size = sizeof d;
     d.batch_size = B; d.head_num = H; d.size_per_head = D; d.total_len = L; d.dtype = dtype; d.nsplit = nsplit;
     return d;
 }
@@ -30,6 +31,7 @@ static fl_attn_io fake_io()
 {
     fl_attn_io io;
     std::memset(&io, 0, sizeof io);
+    io.struct_size = sizeof io;
     void *fake = reinterpret_cast<void *>(0x1000);
     io.q = io.k_new = io.v_new = fake;
     io.k_cache = io.v_cache = fake;
@@ -43,7 +45,7 @@ static fl_attn_io fake_io()
 
 int main()
 {
-    const int Ds[] = {32, 64, 128, 256, 512, 1024};
+    const int Ds[] = {32, 64, 96, 128, 256, 512, 1024};
     const int Ls[] = {1, 2, 63, 64, 65, 1000, 4096, 33100};
     for (int dtype = 0; dtype < 2; ++dtype)
         for (int D : Ds)
@@ -93,7 +95,20 @@ int main()
     fl_attn_desc huge = desc(1, 1, 1024, 2000000, FL_ATTN_F32, 0); // a (b,h) slice beyond 32-bit row offsets
     size_t n = 0;
     EXPECT(fl_decode_attn_workspace_bytes(&huge, &n) == FL_ATTN_ERR_SHAPE);
-    for (int s = 0; s >= -11; --s) EXPECT(fl_attn_strerror(s) != nullptr && std::strlen(fl_attn_strerror(s)) > 0);
+    // struct_size: unset, too small, or from a newer header -> rejected before any member is trusted
+    d = desc(2, 4, 128, 64, FL_ATTN_F16, 0);
+    io = fake_io();
+    d.struct_size = 0;
+    EXPECT(fl_decode_attn_workspace_bytes(&d, &n) == FL_ATTN_ERR_STRUCT_SIZE);
+    d.struct_size = sizeof d + 8;
+    EXPECT(fl_decode_attn_forward(&d, &io, nullptr) == FL_ATTN_ERR_STRUCT_SIZE);
+    d.struct_size = sizeof d;
+    io.struct_size = sizeof io - 8;
+    EXPECT(fl_decode_attn_forward(&d, &io, nullptr) == FL_ATTN_ERR_STRUCT_SIZE);
+    EXPECT(fl_prefill_attn_forward(&d, &io, 8, nullptr) == FL_ATTN_ERR_STRUCT_SIZE);
+    io.struct_size = sizeof io + 16;
+    EXPECT(fl_decode_attn_forward_noalloc(&d, &io, nullptr) == FL_ATTN_ERR_STRUCT_SIZE);
+    for (int s = 0; s >= -12; --s) EXPECT(fl_attn_strerror(s) != nullptr && std::strlen(fl_attn_strerror(s)) > 0);
     std::printf("C-ABI host logic under sanitizers: %d checks, %d failures\n", checks, failures);
     return failures ? 1 : 0;
 }

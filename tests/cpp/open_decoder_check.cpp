@@ -8,6 +8,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <algorithm>
 #include <stdexcept>
 #include <vector>
 
@@ -290,7 +291,7 @@ template <OperationType Op, typename CacheT> static void runAll(const char *tag)
         try { dec.forward(d_from.p, d_freq.p, d_kc.p, d_vc.p, d_dec_out.p, L, 1); } catch (std::runtime_error &) { caught++; }
         try { dec.decodeAttention(d_q.p, d_k.p, d_v.p, (const float *)nullptr, d_kc.p, d_vc.p, d_out.p, P); } catch (std::runtime_error &) { caught++; }
         try {
-            OpenDecoder<Op, OperationType::INT8> bad(B, prompt, gen, H, 96, 4 * HD); // reference: throw "invalid size_per_head!"
+            OpenDecoder<Op, OperationType::INT8> bad(B, prompt, gen, H, 48, 4 * HD); // reference: throw "invalid size_per_head!"
             (void)bad.getWorkspaceSize();
         } catch (std::runtime_error &) { caught++; }
         try {
@@ -304,6 +305,151 @@ template <OperationType Op, typename CacheT> static void runAll(const char *tag)
     HIP_OK(hipStreamDestroy(stream));
 }
 
+// The reference driver's loop (decoding_sampling.cu:232-258): ONE decoder object and ONE workspace serve every layer;
+// initialize(param[layer], buf) is called before every forward() of every step; each layer owns its slice of the K/V
+// cache arena (decoding_sampling.cu:256-257).  One prompt call and `gen_steps` decode steps per layer, with a context
+// split so that the decode steps use the arrival counters in the shared workspace; every quantised output and the
+// final caches of every layer are compared with the oracle run in the same order.
+template <OperationType Op, typename CacheT> static void runLayerLoop(const char *tag)
+{
+    typedef typename DecoderTransformerTraits<Op>::DataType DataT;
+    const int B = 2, H = 4, D = 128, prompt = 24, gen = 8, L = prompt + gen, HD = H * D, layers = 3, gen_steps = 3;
+    const int code = std::is_same<CacheT, float>::value ? 0 : 1;
+    char name[160];
+
+    std::vector<float> freq((size_t)L * D), mask((size_t)L * L);
+    fl_ref_freq_cis(freq.data(), L, D, 10000.0);
+    for (int r = 0; r < L; ++r)
+        for (int c = 0; c < L; ++c) mask[(size_t)r * L + c] = c > r ? -3.4028234664e38f : 0.0f; // samples/llama_fp16.cu:73-81, causal
+    DevBuf<float> d_freq(freq.size()), d_mask(mask.size());
+    d_freq.up(freq.data()); d_mask.up(mask.data());
+
+    const size_t layer_elems = (size_t)B * H * L * D;
+    std::vector<CacheT> kc(layers * layer_elems), vc(kc.size());
+    for (auto &x : kc) x = toCache<CacheT>(frand());
+    for (auto &x : vc) x = toCache<CacheT>(frand());
+    DevBuf<CacheT> d_kc(kc.size()), d_vc(vc.size());
+    d_kc.up(kc.data()); d_vc.up(vc.data());
+
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+    OpenDecoder<Op, OperationType::INT8> dec(B, prompt, gen, H, D, 4 * HD);
+    dec.setContextSplits(2);
+    DevBuf<char> d_ws(dec.getWorkspaceSizeBytes());
+
+    // per-layer parameters: the scales differ per layer, the mask is the one shared array
+    std::vector<std::vector<float>> wq(layers), wk(layers), wv(layers);
+    std::vector<DevBuf<float> *> d_w;
+    std::vector<DecoderInitParam<DataT, int8_t>> param(layers);
+    for (int l = 0; l < layers; ++l) {
+        for (auto *w : {&wq[l], &wk[l], &wv[l]}) {
+            w->resize(HD);
+            for (auto &x : *w) x = 0.01f + 0.01f * (frand() + 1.0f);
+            d_w.push_back(new DevBuf<float>(HD));
+            d_w.back()->up(w->data());
+        }
+        param[l].attn_mask = d_mask.p;
+        param[l].stream = stream;
+        param[l].attention.query_weight.weight_scale = d_w[3 * l]->p;
+        param[l].attention.key_weight.weight_scale = d_w[3 * l + 1]->p;
+        param[l].attention.value_weight.weight_scale = d_w[3 * l + 2]->p;
+    }
+
+    // inputs of every (step, layer): int32 accumulators and activation scales; step 0 is the prompt (24 tokens)
+    const int steps = 1 + gen_steps;
+    auto tokens_of = [&](int step) { return step == 0 ? prompt : 1; };
+    std::vector<std::vector<int32_t>> qi(steps * layers), ki(steps * layers), vi(steps * layers);
+    std::vector<std::vector<float>> sc(steps * layers);
+    std::vector<DevBuf<int32_t> *> d_i;
+    std::vector<DevBuf<float> *> d_s;
+    std::vector<DevBuf<int8_t> *> d_seen8;
+    std::vector<DevBuf<float> *> d_seens;
+    for (int i = 0; i < steps * layers; ++i) {
+        const size_t n = (size_t)B * tokens_of(i / layers) * HD;
+        for (auto *a : {&qi[i], &ki[i], &vi[i]}) {
+            a->resize(n);
+            for (auto &x : *a) x = (int32_t)(frand() * 20000.f);
+            d_i.push_back(new DevBuf<int32_t>(n));
+            d_i.back()->up(a->data());
+        }
+        sc[i].resize((size_t)B * tokens_of(i / layers));
+        for (auto &x : sc[i]) x = 0.002f + 0.001f * (frand() + 1.0f);
+        d_s.push_back(new DevBuf<float>(sc[i].size()));
+        d_s.back()->up(sc[i].data());
+        d_seen8.push_back(new DevBuf<int8_t>(n));
+        d_seens.push_back(new DevBuf<float>(sc[i].size()));
+    }
+
+    DevBuf<DataT> d_from((size_t)B * prompt * HD), d_dec_out((size_t)B * prompt * HD);
+    HookCtx ctx{};
+    ctx.hidden = (size_t)HD;
+    DecoderExternalStages<DataT> st;
+    st.user = &ctx;
+    st.qkv_projection = qkvHook<DataT>;
+    st.post_attention = postHook<DataT>;
+    dec.setExternalStages(st);
+
+    bool classified = false;
+    for (int step = 0; step < steps; ++step) {
+        const int start_pos = step == 0 ? 0 : prompt + step - 1, S = tokens_of(step);
+        for (int l = 0; l < layers; ++l) { // decoding_sampling.cu:242-258
+            const int i = step * layers + l;
+            dec.initialize(param[l], d_ws.p);
+            if (!classified) { // once: the mask is the same array for every layer and call
+                dec.classifyMask();
+                classified = true;
+            }
+            ctx.q = d_i[3 * i]->p; ctx.k = d_i[3 * i + 1]->p; ctx.v = d_i[3 * i + 2]->p;
+            ctx.scale = d_s[i]->p; ctx.seen_int8 = d_seen8[i]->p; ctx.seen_scale = d_seens[i]->p;
+            dec.forward(d_from.p, d_freq.p, d_kc.p + l * layer_elems, d_vc.p + l * layer_elems, d_dec_out.p, start_pos, S);
+        }
+    }
+    HIP_OK(hipStreamSynchronize(stream));
+
+    // the oracle, same order
+    int worst8 = 0;
+    double worst_s = 0;
+    for (int step = 0; step < steps; ++step) {
+        const int start_pos = step == 0 ? 0 : prompt + step - 1, S = tokens_of(step);
+        for (int l = 0; l < layers; ++l) {
+            const int i = step * layers + l;
+            CacheT *kl = kc.data() + l * layer_elems, *vl = vc.data() + l * layer_elems;
+            std::vector<float> want((size_t)B * H * S * D), want_s((size_t)B * S), got_s(want_s.size());
+            std::vector<int8_t> want8((size_t)B * S * HD), got8(want8.size());
+            if (S == 1) {
+                fl_ref_decode_attn_i32(code, B, H, D, L, qi[i].data(), ki[i].data(), vi[i].data(), sc[i].data(), wq[l].data(),
+                                       wk[l].data(), wv[l].data(), kl, vl, freq.data(), -1, mask.data(), L, start_pos, nullptr, -1,
+                                       1.0f / std::sqrt((float)D), want.data(), 1, 1);
+                fl_ref_attn_quantize(B, HD, want.data(), want8.data(), want_s.data());
+            } else {
+                fl_ref_prefill_attn(code, B, H, D, L, S, qi[i].data(), ki[i].data(), vi[i].data(), sc[i].data(), wq[l].data(),
+                                    wk[l].data(), wv[l].data(), kl, vl, freq.data(), -1, mask.data(), L, start_pos,
+                                    1.0f / std::sqrt((float)D), want.data(), 1, 4);
+                fl_ref_attn_quantize_transpose(B, H, S, D, want.data(), want8.data(), want_s.data());
+            }
+            d_seen8[i]->down(got8.data());
+            d_seens[i]->down(got_s.data());
+            for (size_t j = 0; j < want8.size(); ++j) worst8 = std::max(worst8, std::abs((int)got8[j] - (int)want8[j]));
+            for (size_t j = 0; j < want_s.size(); ++j) worst_s = std::fmax(worst_s, std::fabs(got_s[j] - want_s[j]) / want_s[j]);
+        }
+    }
+    std::vector<CacheT> kc_got(kc.size()), vc_got(vc.size());
+    d_kc.down(kc_got.data()); d_vc.down(vc_got.data());
+    std::snprintf(name, sizeof name, "%s layer loop (initialize before every forward): int8 within one step", tag);
+    report(name, worst8 <= 1 && ctx.calls_pre == steps * layers && ctx.calls_post == steps * layers, worst8);
+    std::snprintf(name, sizeof name, "%s layer loop: output scales", tag);
+    report(name, worst_s <= (code ? 1e-3 : 1e-5), worst_s);
+    std::snprintf(name, sizeof name, "%s layer loop: caches of every layer bit-exact", tag);
+    report(name, !std::memcmp(kc_got.data(), kc.data(), kc.size() * sizeof(CacheT)) &&
+                     !std::memcmp(vc_got.data(), vc.data(), vc.size() * sizeof(CacheT)));
+    for (auto *p : d_w) delete p;
+    for (auto *p : d_i) delete p;
+    for (auto *p : d_s) delete p;
+    for (auto *p : d_seen8) delete p;
+    for (auto *p : d_seens) delete p;
+    HIP_OK(hipStreamDestroy(stream));
+}
+
 int main()
 {
     int n = 0;
@@ -314,6 +460,8 @@ int main()
     runAll<OperationType::FP32, float>("OpenDecoder<FP32,INT8>/float-cache");
     runAll<OperationType::FP16, float>("OpenDecoder<FP16,INT8>/float-cache");
     runAll<OperationType::FP16, __half>("OpenDecoder<FP16,INT8>/half-cache");
+    runLayerLoop<OperationType::FP32, float>("OpenDecoder<FP32,INT8>/float-cache");
+    runLayerLoop<OperationType::FP16, __half>("OpenDecoder<FP16,INT8>/half-cache");
     std::printf(g_fail ? "SOME CHECKS FAILED\n" : "ALL CHECKS PASSED\n");
     return g_fail;
 }

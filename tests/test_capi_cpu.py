@@ -39,20 +39,22 @@ def test_header_and_binding_agree_and_library_exports_everything():
 
 
 def test_struct_layouts_match_the_header():
-    # natural alignment on x86-64: 8 x 4 bytes, and 10 pointers/size_t + int64 + 4 x int32 + 7 pointers
-    assert C.sizeof(capi.AttnDesc) == 32
-    assert C.sizeof(capi.AttnIO) == 10 * 8 + 8 + 8 + 16 + 7 * 8
+    # natural alignment on x86-64: 9 x 4 bytes; struct_size (padded to 8) + 10 pointers + size_t + int64 + 4 x int32 + 7 pointers
+    assert C.sizeof(capi.AttnDesc) == 36
+    assert C.sizeof(capi.AttnIO) == 8 + 10 * 8 + 8 + 8 + 16 + 7 * 8
+    assert desc().struct_size == 36 and fake_io().struct_size == C.sizeof(capi.AttnIO)
     assert C.sizeof(capi.AttnPlan) == 16
 
 
 def test_strerror_covers_every_status():
-    msgs = {capi.strerror(s) for s in range(0, -11, -1)}
-    assert len(msgs) == 11 and "unknown status" not in msgs
+    msgs = {capi.strerror(s) for s in range(0, -12, -1)}
+    assert len(msgs) == 12 and "unknown status" not in msgs
     assert capi.strerror(-99) == "unknown status"
 
 
 @pytest.mark.parametrize("kw,want", [
-    (dict(D=96), capi.FL_ATTN_ERR_HEAD_DIM),      # reference: throw "invalid size_per_head!"
+    (dict(D=48), capi.FL_ATTN_ERR_HEAD_DIM),      # reference: throw "invalid size_per_head!" (decoder_kernels.cu:588)
+    (dict(D=160), capi.FL_ATTN_ERR_HEAD_DIM),
     (dict(D=2048), capi.FL_ATTN_ERR_HEAD_DIM),
     (dict(D=0), capi.FL_ATTN_ERR_HEAD_DIM),
     (dict(B=0), capi.FL_ATTN_ERR_SHAPE),
@@ -73,6 +75,38 @@ def test_descriptor_validation(kw, want):
     d = desc(**kw)
     assert lib.fl_decode_attn_workspace_bytes(C.byref(d), C.byref(n)) == want
     assert lib.fl_decode_attn_forward(C.byref(d), C.byref(fake_io()), None) == want
+
+
+def test_struct_size_is_checked_before_any_member_is_trusted():
+    """A caller built against another header: struct_size unset, shorter than the first layout that has it, or
+    larger than the library's own struct."""
+    lib = capi.load()
+    n = C.c_size_t(0)
+    for bad in (0, 32, C.sizeof(capi.AttnDesc) + 4):
+        d = desc()
+        d.struct_size = bad
+        assert lib.fl_decode_attn_workspace_bytes(C.byref(d), C.byref(n)) == capi.FL_ATTN_ERR_STRUCT_SIZE
+        assert lib.fl_prefill_attn_workspace_bytes(C.byref(d), 8, C.byref(n)) == capi.FL_ATTN_ERR_STRUCT_SIZE
+        assert lib.fl_decode_attn_forward(C.byref(d), C.byref(fake_io()), None) == capi.FL_ATTN_ERR_STRUCT_SIZE
+    for bad in (0, C.sizeof(capi.AttnIO) - 8, C.sizeof(capi.AttnIO) + 8):
+        io = fake_io(start_pos=64)  # would be FL_ATTN_ERR_POSITION with a good struct_size
+        io.struct_size = bad
+        assert lib.fl_decode_attn_forward(C.byref(desc()), C.byref(io), None) == capi.FL_ATTN_ERR_STRUCT_SIZE
+        assert lib.fl_decode_attn_forward_noalloc(C.byref(desc()), C.byref(io), None) == capi.FL_ATTN_ERR_STRUCT_SIZE
+        assert lib.fl_prefill_attn_forward(C.byref(desc()), C.byref(io), 8, None) == capi.FL_ATTN_ERR_STRUCT_SIZE
+    assert lib.fl_decode_attn_forward(C.byref(desc()), C.byref(fake_io(start_pos=64)), None) == capi.FL_ATTN_ERR_POSITION
+
+
+def test_cache_slices_stay_below_two_gib():
+    """The streaming kernel's buffer descriptors span 2^31 bytes from the base of a (batch, head) slice."""
+    lib = capi.load()
+    n = C.c_size_t(0)
+    ok = desc(B=1, H=1, D=128, L=(1 << 31) // 256 - 65, dtype=capi.FL_ATTN_F16)
+    assert lib.fl_decode_attn_workspace_bytes(C.byref(ok), C.byref(n)) == 0
+    too_long = desc(B=1, H=1, D=128, L=(1 << 31) // 256 - 64, dtype=capi.FL_ATTN_F16)
+    assert lib.fl_decode_attn_workspace_bytes(C.byref(too_long), C.byref(n)) == capi.FL_ATTN_ERR_SHAPE
+    assert lib.fl_decode_attn_workspace_bytes(C.byref(desc(B=1, H=1, D=128, L=(1 << 31) // 512, dtype=capi.FL_ATTN_F32)),
+                                              C.byref(n)) == capi.FL_ATTN_ERR_SHAPE
 
 
 def test_null_arguments():

@@ -19,7 +19,7 @@ def test_open_decoder_cpp_driver(gpu):
     print(res.stdout)
     assert res.returncode == 0, res.stdout
     assert "ALL CHECKS PASSED" in res.stdout
-    assert res.stdout.count("PASS ") == 30 and "FAIL" not in res.stdout
+    assert res.stdout.count("PASS ") == 36 and "FAIL" not in res.stdout
 
 
 def test_open_decoder_library_exports_the_reference_instantiations():

@@ -117,7 +117,7 @@ def test_ctx1_is_exactly_v_new(gpu):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
-@pytest.mark.parametrize("D", [32, 64, 128, 256, 512, 1024])
+@pytest.mark.parametrize("D", [32, 64, 96, 128, 256, 512, 1024])
 def test_head_sizes(gpu, dtype, D):
     c = Case(2, 2, D, 300, dtype, start_pos=277, seed=D)
     check(c, gpu, what=f"D={D}")
@@ -291,7 +291,7 @@ def test_forward_reports_errors_instead_of_exiting(gpu):
         op.forward(q, q, q, kc.view(-1)[1:], kc, f, start_pos=3)
     assert e.value.status == capi.FL_ATTN_ERR_ALIGNMENT
     with pytest.raises(capi.FlAttnError) as e:
-        DecodeAttention(2, 4, 96, 64, torch.float16, device=gpu)
+        DecodeAttention(2, 4, 48, 64, torch.float16, device=gpu)  # the reference rejects it too (decoder_kernels.cu:564-588)
     assert e.value.status == capi.FL_ATTN_ERR_HEAD_DIM
     out = op.forward(q, q, q, kc, kc, f, start_pos=3)  # still usable afterwards
     torch.cuda.synchronize()

@@ -24,12 +24,9 @@ def make(B, H, D, L, S, dtype, seed=11):
     return q, k, v, kc, vc, synth.freq_cis_table(L, D)
 
 
-_last = {}
-
-
-def close(out, want, dtype, what, rows=slice(None)):
-    """assert_out_close with the float oracle of the last run_both at hand for FP32 caches."""
-    fr = _last.get("float_ref") if dtype == "f32" else None
+def close(out, want, dtype, what, run, rows=slice(None)):
+    """assert_out_close with the float oracle of the same run_both call (its third result) at hand for FP32 caches."""
+    fr = run.float_ref if dtype == "f32" else None
     return assert_out_close(out, want, dtype, what, float_ref=None if fr is None else (lambda: fr()[:, :, rows]))
 
 
@@ -44,7 +41,7 @@ def run_both(gpu, B, H, D, L, S, P, dtype, mask=None, rope_row=-1, pad_nan=True,
     want = ref.prefill_attn(q, k, v, kc_ref, vc_ref, f, start_pos=P, rope_row=rope_row, attn_mask=mask,
                             acc_double=True, threads=16)
     # the same inputs through the oracle's float arithmetic (sequential FP32 sums), evaluated on demand
-    _last["float_ref"] = lambda: ref.prefill_attn(q, k, v, kc.copy(), vc.copy(), f, start_pos=P, rope_row=rope_row,
+    float_ref = lambda: ref.prefill_attn(q, k, v, kc.copy(), vc.copy(), f, start_pos=P, rope_row=rope_row,
                                                   attn_mask=mask, acc_double=False, threads=16)
     t = lambda a: None if a is None else torch.from_numpy(a).to(gpu)
     op = PrefillAttention(B, H, D, L, S, torch.float16 if dtype == "f16" else torch.float32, device=gpu)
@@ -55,6 +52,7 @@ def run_both(gpu, B, H, D, L, S, P, dtype, mask=None, rope_row=-1, pad_nan=True,
     # rows past the prompt were NaN before and must still be: compare bit patterns of everything
     assert_cache_bit_exact(kc_g, kc_ref, "k_cache")
     assert_cache_bit_exact(vc_g, vc_ref, "v_cache")
+    op.float_ref = float_ref
     return out.cpu().numpy(), want, op
 
 
@@ -63,16 +61,16 @@ def run_both(gpu, B, H, D, L, S, P, dtype, mask=None, rope_row=-1, pad_nan=True,
                                  (50, 37), (1, 200), (64, 64)])
 def test_prefill_matches_oracle(gpu, dtype, S, P):
     L = 512
-    out, want, _ = run_both(gpu, 2, 3, 128, L, S, P, dtype, mask=causal_mask(L), seed=S + P)
-    close(out, want, dtype, f"S={S} P={P}")
+    out, want, run = run_both(gpu, 2, 3, 128, L, S, P, dtype, mask=causal_mask(L), seed=S + P)
+    close(out, want, dtype, f"S={S} P={P}", run=run)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
-@pytest.mark.parametrize("D", [32, 64, 128, 256, 512, 1024])
+@pytest.mark.parametrize("D", [32, 64, 96, 128, 256, 512, 1024])
 def test_prefill_head_sizes_and_no_mask(gpu, dtype, D):
     # the reference's set of head sizes (decoder_kernels.cu:474-551, :588), plus 32
-    out, want, _ = run_both(gpu, 2, 5, D, 256, 77, 10, dtype, mask=None, seed=D)
-    close(out, want, dtype, f"D={D} no mask")
+    out, want, run = run_both(gpu, 2, 5, D, 256, 77, 10, dtype, mask=None, seed=D)
+    close(out, want, dtype, f"D={D} no mask", run=run)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
@@ -83,8 +81,8 @@ def test_prefill_wide_heads_with_masks(gpu, dtype, D, S, P):
     blocks, chunked prompts, the -1e5 causal mask (every tile evaluated) and the -FLT_MAX one (tiles dropped)."""
     L = 256
     for fill in (-1e5, -FMAX):
-        out, want, _ = run_both(gpu, 2, 3, D, L, S, P, dtype, mask=causal_mask(L, fill), seed=D + S + P)
-        close(out, want, dtype, f"D={D} S={S} P={P} fill={fill}")
+        out, want, run = run_both(gpu, 2, 3, D, L, S, P, dtype, mask=causal_mask(L, fill), seed=D + S + P)
+        close(out, want, dtype, f"D={D} S={S} P={P} fill={fill}", run=run)
 
 
 def test_prefill_wide_heads_dense_mask_scaled_keys_and_decode_handover(gpu):
@@ -123,9 +121,9 @@ def test_prefill_strict_mask_first_row_is_nan(gpu):
     L = 64
     fm = np.finfo(np.float32).max
     m = np.where(np.arange(L)[:, None] > np.arange(L)[None, :], 0.0, -fm).astype(np.float32)
-    out, want, _ = run_both(gpu, 1, 2, 64, L, 40, 0, "f32", mask=m)
+    out, want, run = run_both(gpu, 1, 2, 64, L, 40, 0, "f32", mask=m)
     assert np.isnan(want[:, :, 0]).all() and np.isnan(out[:, :, 0]).all()
-    close(out[:, :, 1:], want[:, :, 1:], "f32", "strict mask rows 1..", rows=slice(1, None))
+    close(out[:, :, 1:], want[:, :, 1:], "f32", "strict mask rows 1..", rows=slice(1, None), run=run)
 
 
 FMAX = float(np.finfo(np.float32).max)
@@ -137,16 +135,16 @@ def test_prefill_causal_mask_with_flt_max(gpu, dtype, S, P):
     """The reference driver's mask value (samples/llama_fp16.cu:73-81): fully masked tiles contribute exact zeros
     whether a kernel evaluates or drops them."""
     L = 512
-    out, want, _ = run_both(gpu, 2, 3, 128, L, S, P, dtype, mask=causal_mask(L, -FMAX), seed=3 * S + P)
-    close(out, want, dtype, f"-FLT_MAX causal S={S} P={P}")
+    out, want, run = run_both(gpu, 2, 3, 128, L, S, P, dtype, mask=causal_mask(L, -FMAX), seed=3 * S + P)
+    close(out, want, dtype, f"-FLT_MAX causal S={S} P={P}", run=run)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
 @pytest.mark.parametrize("D", [32, 64])
 def test_prefill_small_heads_with_causal_mask(gpu, dtype, D):
     L = 320
-    out, want, _ = run_both(gpu, 2, 4, D, L, 200, 100, dtype, mask=causal_mask(L, -FMAX), seed=D + 1)
-    close(out, want, dtype, f"D={D} -FLT_MAX causal")
+    out, want, run = run_both(gpu, 2, 4, D, L, 200, 100, dtype, mask=causal_mask(L, -FMAX), seed=D + 1)
+    close(out, want, dtype, f"D={D} -FLT_MAX causal", run=run)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
@@ -197,7 +195,7 @@ def test_prefill_fast_qk_meets_the_bar_on_ordinary_data(gpu):
 def test_prefill_strict_mask_first_row_is_nan_f16(gpu):
     L = 192
     m = np.where(np.arange(L)[:, None] > np.arange(L)[None, :], 0.0, -FMAX).astype(np.float32)
-    out, want, _ = run_both(gpu, 1, 2, 128, L, 150, 0, "f16", mask=m)
+    out, want, run = run_both(gpu, 1, 2, 128, L, 150, 0, "f16", mask=m)
     assert np.isnan(want[:, :, 0]).all() and np.isnan(out[:, :, 0]).all()
     assert not np.isnan(out[:, :, 1:]).any()
     assert_out_close(out[:, :, 1:], want[:, :, 1:], "f16", "strict mask rows 1.. (f16)")
@@ -209,7 +207,7 @@ def test_prefill_sliding_window_mask_f16(gpu, fill):
     L, S, P, win = 640, 200, 400, 96
     i, j = np.arange(L)[:, None], np.arange(L)[None, :]
     m = np.where((j > i) | (j < i - win), fill, 0.0).astype(np.float32)
-    out, want, _ = run_both(gpu, 2, 2, 128, L, S, P, "f16", mask=m, seed=5)
+    out, want, run = run_both(gpu, 2, 2, 128, L, S, P, "f16", mask=m, seed=5)
     assert_out_close(out, want, "f16", f"sliding window fill={fill}")
 
 
@@ -287,14 +285,14 @@ def test_prefill_hip_graph_replay_matches_eager(gpu):
 
 def test_prefill_literal_rope_rows(gpu):
     # reference as written: token s of the prompt is rotated by table row s (decoder_kernels.cu:440)
-    out, want, _ = run_both(gpu, 2, 4, 128, 128, 60, 20, "f32", mask=causal_mask(128), rope_row=0)
-    close(out, want, "f32", "rope_row=0")
+    out, want, run = run_both(gpu, 2, 4, 128, 128, 60, 20, "f32", mask=causal_mask(128), rope_row=0)
+    close(out, want, "f32", "rope_row=0", run=run)
 
 
 def test_prefill_llama7b_shape(gpu):
     # B=4, 32 heads, D=128, prompt of 512 tokens, fp16 caches
     L = 640
-    out, want, _ = run_both(gpu, 4, 32, 128, L, 512, 0, "f16", mask=causal_mask(L))
+    out, want, run = run_both(gpu, 4, 32, 128, L, 512, 0, "f16", mask=causal_mask(L))
     assert_out_close(out, want, "f16", "7B prompt 512")
 
 
@@ -462,7 +460,7 @@ def test_prefill_argument_errors(gpu):
     import torch
     from fasterllama_amd.decode_attn import PrefillAttention
     with pytest.raises(capi.FlAttnError) as e:
-        PrefillAttention(1, 2, 96, 64, 16, torch.float16, device=gpu)
+        PrefillAttention(1, 2, 48, 64, 16, torch.float16, device=gpu)
     assert e.value.status == capi.FL_ATTN_ERR_HEAD_DIM
     op = PrefillAttention(1, 2, 64, 64, 16, torch.float16, device=gpu)
     z = torch.zeros(1, 16, 2, 64, dtype=torch.float16, device=gpu)

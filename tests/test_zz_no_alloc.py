@@ -40,6 +40,41 @@ def test_noalloc_ragged_forced_splits_and_unsplit(gpu, dtype):
     both(Case(2, 4, 64, 256, dtype, start_pos=100), gpu, nsplit=1)  # no scratch needed at all
 
 
+def test_noalloc_counters_keep_their_place_across_shapes(gpu):
+    """The arrival counters own a fixed part of the scratch array: a call with few (batch, head) pairs that writes
+    floats into the array (an INT8-only step keeps its float output there; a split step its partials) must not leave
+    non-zero words where a later split step with more pairs keeps its counters."""
+    import torch
+    from fasterllama_amd.decode_attn import DecodeAttention
+    # 1. INT8-only, unsplit, B*H = 32: the float output [32, 128] goes through the scratch array
+    c1 = Case(1, 32, 128, 512, "f16", start_pos=300, seed=3)
+    t = lambda a: torch.from_numpy(a).to(gpu)
+    op1 = DecodeAttention(1, 32, 128, 512, torch.float16, nsplit=1, device=gpu)
+    res = {}
+    for entry in ("forward", "noalloc"):
+        q8 = torch.zeros(1, 32 * 128, dtype=torch.int8, device=gpu)
+        sc = torch.zeros(1, dtype=torch.float32, device=gpu)
+        io = op1.make_io(t(c1.q), t(c1.k_new), t(c1.v_new), t(c1.k_cache), t(c1.v_cache), t(c1.freq), None,
+                         start_pos=300, out_int8=q8, out_scale=sc)
+        if entry == "noalloc":
+            io.workspace, io.workspace_bytes = None, 0
+            capi.check(op1.launch_noalloc(io))
+        else:
+            capi.check(op1.launch(io))
+        torch.cuda.synchronize()
+        res[entry] = (q8.cpu().numpy(), sc.cpu().numpy())
+    assert np.array_equal(res["forward"][0], res["noalloc"][0]) and np.array_equal(res["forward"][1], res["noalloc"][1])
+    assert np.abs(res["noalloc"][0]).max() == 127
+    # 2. a tiny split step: its partials sit at the start of the array
+    both(Case(1, 2, 32, 512, "f32", start_pos=400, seed=4), gpu, nsplit=4)
+    # 3. split steps with more pairs, merged inside the launch: B*H = 128 and 200 counters
+    op = both(Case(4, 32, 128, 2048, "f16", start_pos=2047, seed=5), gpu)
+    plan = op.plan(2048)
+    assert plan.nsplit > 1 and plan.two_pass == 2
+    both(Case(5, 40, 64, 1024, "f32", start_pos=1000, seed=6), gpu, nsplit=3)
+    both(Case(4, 32, 128, 2048, "f16", start_pos=2047, seed=7), gpu)
+
+
 def test_noalloc_rejects_what_does_not_fit(gpu):
     import ctypes as C
     import torch
