@@ -599,6 +599,7 @@ void prefill_attn_kernel(const PrefillParams p)
 // One 32-bit word per (128-query block, key tile): byte w is the class of the block's w-th wave.
 constexpr float kMaskedBelow = -1e30f;
 constexpr float kLazyMax = 8.0f; // base-2 units
+constexpr float kPairLogit = 4.0f; // fp16 prompt kernel: scores (after scaling, natural units) above which the query remainders are multiplied in
 
 // grid = (key tiles, query blocks), block = 256.
 __global__ __launch_bounds__(256) void prefill_mask_classify_kernel(const PrefillParams p, int NT)
@@ -1014,6 +1015,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         else return lds_read_tr16(&sV[buf][row0 + vrow][32 * dt + vcol]);
     };
     const float inv_scale = 1.0f / p.scale;
+    const float pair_raw = kPairLogit * inv_scale; // the remainder product's threshold in units of the raw products
     const bool mask_vec4 = HAS_MASK && (p.mask_ld & 3) == 0 && (reinterpret_cast<uintptr_t>(p.attn_mask) & 15u) == 0;
 
     // The rotated queries must have landed before the loop: a wait inside it would also wait for
@@ -1124,17 +1126,11 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                     for (int v = 0; v < 16; ++v) zero[v] = 0.f;
                     st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka0, qreg[0], zero, 0, 0, 0); // the literal 0 operand
                 }
-                // With QSPLIT every K operand multiplies the query's fp16 value and its remainder: the pair
-                // carries 22 significant bits, so the scores keep FP32-level accuracy at any magnitude
-                // (a single fp16 query leaves |s| * 2^-12 of error in each score).
-                if constexpr (QSPLIT) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka0, qlo[0], st, 0, 0, 0);
 #pragma unroll
                 for (int c = 1; c < NC; ++c) {
                     const half8 ka = PF_KA ? kall[PF_KA ? c : 0] : k_operand(buf, c);
                     st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[c], st, 0, 0, 0);
-                    if constexpr (QSPLIT) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qlo[c], st, 0, 0, 0);
                 }
-
                 half4 vlo[PF_VA ? NDT : 1][2], vhi[PF_VA ? NDT : 1][2];
                 if constexpr (PF_VA) {
 #pragma unroll
@@ -1161,6 +1157,25 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                     v_stage(0, 0);
                     __builtin_amdgcn_sched_barrier(0);
                 }
+                // With QSPLIT the K operands also multiply the queries' remainders q - fp16(q): the pair carries
+                // 22 significant bits, so the scores keep FP32-level accuracy at any magnitude (a single fp16
+                // query leaves about |s| * 2^-12 of error in a score s).  The remainder product is additive, so it
+                // is issued only where it can matter: when some score of the wave's tile exceeds kPairLogit in
+                // magnitude after scaling (wave-uniform test on the first product; a NaN or an infinity, e.g. the
+                // -inf of keys past the context, takes the full path).  Below that the skipped term is under
+                // kPairLogit * 2^-12 ~ 1e-3 relative in a weight at the very worst and ~1.5e-4 typically, the
+                // size of the rounding of the weights to fp16 that every tile carries anyway.
+                if constexpr (QSPLIT) {
+                    float am = fmaxf(fmaxf(fabsf(st[0]), fabsf(st[1])), fabsf(st[2]));
+#pragma unroll
+                    for (int v = 3; v < 15; v += 2) am = fmaxf(fmaxf(am, fabsf(st[v])), fabsf(st[v + 1]));
+                    am = fmaxf(am, fabsf(st[15]));
+                    if (__ballot(!(am <= pair_raw)) != 0ull) {
+#pragma unroll
+                        for (int c = 0; c < NC; ++c) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kall[PF_KA ? c : 0], qlo[c], st, 0, 0, 0);
+                    }
+                }
+
                 // Softmax update of this lane's query (decoder_kernels.cu:811-833 in base 2).  The reference
                 // maximum m may lag the true running maximum by up to kLazyMax (weights up to 2^kLazyMax,
                 // well inside fp16 and exact in the final ratio): with 32 queries per wave some maximum
