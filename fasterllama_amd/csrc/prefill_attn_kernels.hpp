@@ -184,7 +184,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int kPrefillQueriesPerBlock = 128; // 4 waves x 32 queries
 constexpr int kPrefillKeysPerStep = 32;
-constexpr uint32_t kTileSkip = 0, kTileZero = 1, kTileMixed = 2; // mask tile classes, see prefill_mask_classify_kernel
+constexpr uint32_t kTileSkip = 0, kTileZero = 1, kTileMixed = 2, kTileDiag = 3; // mask tile classes, see prefill_mask_classify_kernel
 
 // Classes of key tile t for the four 32-query sub-blocks of 128-query block qb, one per byte: from the words
 // this call's classify kernel wrote, or from the caller's persistent table over the whole mask (one byte per
@@ -485,7 +485,7 @@ void prefill_attn_kernel(const PrefillParams p)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int key = k0 + 8 * (v / 4) + 4 * hf + (v % 4);
-            mk[v] = (HAS_MASK && tc == kTileMixed && key < ctx) ? mrow[key] : 0.f;
+            mk[v] = (HAS_MASK && tc >= kTileMixed && key < ctx) ? mrow[key] : 0.f; // (a DIAG tile is read like a MIXED one here)
         }
     };
 
@@ -595,11 +595,24 @@ void prefill_attn_kernel(const PrefillParams p)
 //          exactly 0, so the tile contributes exact zeros to the sum and the output — skipping it
 //          is bit-identical to evaluating it (decoder_kernels.cu:811-833 arithmetic);
 //   ZERO   drop the mask term where all entries are +-0 (fma(s, scale, 0) == s*scale);
-//   MIXED  evaluate the general form.
+//   MIXED  evaluate the general form;
+//   DIAG   the diagonal tile of a causal mask, whole inside the prompt and the context: +-0 where the key's
+//          place in the tile is at or before the query's, <= -1e30 after it.  The fp16 kernel builds such a
+//          tile's term from lane indices (-inf for the masked entries: exp gives the same exact 0, and the
+//          tile's own diagonal keeps every row's maximum finite) and never reads the mask under the usual
+//          causal mask; the other kernels read it like a MIXED tile.
 // One 32-bit word per (128-query block, key tile): byte w is the class of the block's w-th wave.
 constexpr float kMaskedBelow = -1e30f;
 constexpr float kLazyMax = 8.0f; // base-2 units
 constexpr float kPairLogit = 4.0f; // fp16 prompt kernel: scores (after scaling, natural units) above which the query remainders are multiplied in
+
+// Class of a wave's 32 x 32 tile from its lanes' findings (each lane has looked at 16 entries of one column).
+__device__ __forceinline__ uint32_t classify_ballots(bool open, bool nonzero, bool diag)
+{
+    if (__ballot(open) == 0ull) return kTileSkip;
+    if (__ballot(nonzero) == 0ull) return kTileZero;
+    return __ballot(!diag) == 0ull ? kTileDiag : kTileMixed;
+}
 
 // grid = (key tiles, query blocks), block = 256.
 __global__ __launch_bounds__(256) void prefill_mask_classify_kernel(const PrefillParams p, int NT)
@@ -615,14 +628,16 @@ __global__ __launch_bounds__(256) void prefill_mask_classify_kernel(const Prefil
         const int col = min(t * kPrefillKeysPerStep + (lane & 31), ctx - 1);
         uint32_t nonzero = 0;
         bool open = false;
+        bool diag = q0 + 32 <= p.S && (t + 1) * kPrefillKeysPerStep <= ctx; // no repeated row or column
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
             const int q = min(q0 + 2 * j + (lane >> 5), p.S - 1);
             const float v = p.attn_mask[(size_t)(p.start_pos + q) * p.mask_ld + col];
             nonzero |= __float_as_uint(v) << 1; // the sign is shifted out: -0 counts as zero
             open |= !(v <= kMaskedBelow);       // a NaN entry keeps the tile
+            diag &= (lane & 31) <= 2 * j + (lane >> 5) ? (__float_as_uint(v) << 1) == 0u : v <= kMaskedBelow;
         }
-        cls = __ballot(open) == 0ull ? kTileSkip : (__ballot(nonzero != 0u) == 0ull ? kTileZero : kTileMixed);
+        cls = classify_ballots(open, nonzero != 0u, diag);
     }
     if (lane == 0) s_cls[wave] = cls;
     __syncthreads();
@@ -639,14 +654,16 @@ __global__ __launch_bounds__(64) void mask_class_table_kernel(const float *mask,
     const int col = min(t * kPrefillKeysPerStep + (lane & 31), cols - 1);
     uint32_t nonzero = 0;
     bool open = false;
+    bool diag = rb * 32 + 32 <= rows && (t + 1) * kPrefillKeysPerStep <= cols; // no repeated row or column
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
         const int r = min(rb * 32 + 2 * j + (lane >> 5), rows - 1);
         const float v = mask[(size_t)r * mask_ld + col];
         nonzero |= __float_as_uint(v) << 1; // the sign is shifted out: -0 counts as zero
         open |= !(v <= kMaskedBelow);       // a NaN entry keeps the tile
+        diag &= (lane & 31) <= 2 * j + (lane >> 5) ? (__float_as_uint(v) << 1) == 0u : v <= kMaskedBelow;
     }
-    const uint32_t cls = __ballot(open) == 0ull ? kTileSkip : (__ballot(nonzero != 0u) == 0ull ? kTileZero : kTileMixed);
+    const uint32_t cls = classify_ballots(open, nonzero != 0u, diag);
     if (lane == 0) table[(size_t)t * table_ld + rb] = (uint8_t)cls;
 }
 
@@ -1063,12 +1080,16 @@ void prefill_attn_f16_kernel(const PrefillParams p)
             const int k0 = t * BN;
             uint32_t tc = kTileZero;
             if constexpr (HAS_MASK) tc = __builtin_amdgcn_readfirstlane((e0 >> (2 * wave)) & 3u);
-            const bool special = tc != kTileSkip && (k0 + BN > ctx || tc == kTileMixed);
+            const bool special = tc != kTileSkip && (k0 + BN > ctx || tc >= kTileMixed);
             floatx16 st;
             if (special) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) st[v] = 0.f;
                 if constexpr (HAS_MASK) {
+                    if (tc == kTileDiag) { // keys after the query's place in the tile are masked: no memory access
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) st[v] = 8 * (v / 4) + 4 * hf + (v % 4) > qi ? -__builtin_inff() : 0.f;
+                    }
                     if (tc == kTileMixed) {
                         // Mask entries of this lane's query, straight into the score layout (four runs of
                         // four keys).  Only tiles that straddle a mask boundary come here — the diagonal
@@ -1160,19 +1181,19 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 // With QSPLIT the K operands also multiply the queries' remainders q - fp16(q): the pair carries
                 // 22 significant bits, so the scores keep FP32-level accuracy at any magnitude (a single fp16
                 // query leaves about |s| * 2^-12 of error in a score s).  The remainder product is additive, so it
-                // is issued only where it can matter: when some score of the wave's tile exceeds kPairLogit in
-                // magnitude after scaling (wave-uniform test on the first product; a NaN or an infinity, e.g. the
-                // -inf of keys past the context, takes the full path).  Below that the skipped term is under
-                // kPairLogit * 2^-12 ~ 1e-3 relative in a weight at the very worst and ~1.5e-4 typically, the
-                // size of the rounding of the weights to fp16 that every tile carries anyway.
+                // is issued only where it can matter: when the largest score of some query in the wave's tile
+                // exceeds kPairLogit in magnitude after scaling (wave-uniform test on the maximum the softmax needs
+                // anyway; a NaN, or a query whose keys are all masked, takes the full path).  A score s below its
+                // query's maximum M enters the output with weight w = e^(s - M) <= 1 and relative error |s| * 2^-12;
+                // with |M| <= kPairLogit that is at most kPairLogit * 2^-12 ~ 1e-3 of a weight at the very worst
+                // (for s < -kPairLogit, |s| * e^(s - M) <= |s| * e^(s + kPairLogit) <= kPairLogit) and ~1.5e-4
+                // typically, the size of the rounding of the weights to fp16 that every tile carries anyway.
+                float mxq = cross_half_max(max16(st)); // raw units
                 if constexpr (QSPLIT) {
-                    float am = fmaxf(fmaxf(fabsf(st[0]), fabsf(st[1])), fabsf(st[2]));
-#pragma unroll
-                    for (int v = 3; v < 15; v += 2) am = fmaxf(fmaxf(am, fabsf(st[v])), fabsf(st[v + 1]));
-                    am = fmaxf(am, fabsf(st[15]));
-                    if (__ballot(!(am <= pair_raw)) != 0ull) {
+                    if (__ballot(!(fabsf(mxq) <= pair_raw)) != 0ull) {
 #pragma unroll
                         for (int c = 0; c < NC; ++c) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kall[PF_KA ? c : 0], qlo[c], st, 0, 0, 0);
+                        mxq = cross_half_max(max16(st));
                     }
                 }
 
@@ -1181,7 +1202,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 // well inside fp16 and exact in the final ratio): with 32 queries per wave some maximum
                 // moves in almost every tile, and rescaling 64 accumulators each time would cost as much
                 // vector time as the softmax itself.
-                const float mx = fmaxf(m, cross_half_max(max16(st)) * scale);
+                const float mx = fmaxf(m, mxq * scale);
                 if (__ballot(mx > m + kLazyMax) != 0ull) { // wave-uniform
                     const float alpha = __builtin_amdgcn_exp2f(m - mx);
                     m = mx;
@@ -1391,7 +1412,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void prefill_attn_wide_kernel(cons
         }
         // v = qk * scale + mask (decoder_kernels.cu:815); fma(s, scale, 0) == s * scale, so tiles whose mask
         // entries are all zero take the short way
-        if (HAS_MASK && tc == kTileMixed) {
+        if (HAS_MASK && tc >= kTileMixed) { // (a DIAG tile is read like a MIXED one here)
 #pragma unroll
             for (int v = 0; v < 16; ++v) sc[v] = fmaf(sc[v], scale, mrow[min(k0 + 8 * (v / 4) + 4 * hf + (v % 4), ctx - 1)]);
         } else {

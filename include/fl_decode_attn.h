@@ -209,8 +209,8 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int3
                             void *hip_stream);
 
 /* The mask of the reference is one [L, L] array that every layer and every call reuses
- * (samples/llama_fp16.cu:139-150), so its 32 x 32 tiles can be classified (all <= -1e30 / all zero / mixed)
- * once: fl_prefill_mask_classify writes one byte per tile (fl_prefill_mask_classes_bytes bytes: key tile t, row
+ * (samples/llama_fp16.cu:139-150), so its 32 x 32 tiles can be classified (all <= -1e30 / all zero / the
+ * diagonal tile of a causal mask / anything else) once: fl_prefill_mask_classify writes one byte per tile (fl_prefill_mask_classes_bytes bytes: key tile t, row
  * block r at t * ld + r, n = ceil(L/32), ld = n rounded up to a multiple of 4; the table must be 4-byte aligned),
  * for a mask with total_len rows and columns and row stride mask_ld >= total_len.  A prompt-phase call whose
  * io.mask_tile_classes points at that table, with the same attn_mask and mask_ld and a start_pos that is a

@@ -449,11 +449,16 @@ def test_prefill_with_a_persistent_mask_class_table(gpu, dtype, D):
             assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32)), f"{name} S={S} P={P}"
             assert_out_close(outs[1], want, dtype, f"class table, {name} S={S} P={P}",
                              float_ref=lambda: ref.prefill_attn(q, k, v, kc.copy(), vc.copy(), f, start_pos=P, attn_mask=m, threads=16))
-    # the table itself: 0 = every entry <= -1e30, 1 = every entry zero, 2 = anything else
+    # the table itself: 0 = every entry <= -1e30, 1 = every entry zero, 3 = the diagonal tile of a causal mask (zero
+    # up to the row's own place in the tile, <= -1e30 after it), 2 = anything else
     # layout: byte [key tile][row block], rows padded to a multiple of four row blocks
     tab = op.classify_mask(t(masks["causal -FLT_MAX"].astype(np.float32))).cpu().numpy().reshape(10, 12)[:, :10].T
-    assert (np.diag(tab) == 2).all() and (np.tril(tab, -1)[np.tril_indices(10, -1)] == 1).all() \
+    assert (np.diag(tab) == 3).all() and (np.tril(tab, -1)[np.tril_indices(10, -1)] == 1).all() \
         and (tab[np.triu_indices(10, 1)] == 0).all()
+    tab = op.classify_mask(t(masks["causal -1e5"].astype(np.float32))).cpu().numpy().reshape(10, 12)[:, :10].T
+    assert (np.diag(tab) == 2).all() and (tab[np.triu_indices(10, 1)] == 2).all()  # -1e5 is not provably zero weight
+    tab = op.classify_mask(t(masks["window 70"].astype(np.float32))).cpu().numpy().reshape(10, 12)[:, :10].T
+    assert (np.diag(tab) == 3).all() and (tab[np.arange(4, 10), np.arange(0, 6)] == 0).all()
 
 
 def test_prefill_argument_errors(gpu):
