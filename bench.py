@@ -470,6 +470,7 @@ def calibrate(args) -> int:
     lib.fl_calib_empty.argtypes = [C.c_void_p]
     lib.fl_calib_stream_read_two.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_void_p]
     lib.fl_calib_coexec.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    lib.fl_calib_attn_loop.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     dev = torch.device("cuda:0")
     stream = torch.cuda.current_stream(dev)
     sp = C.c_void_p(stream.cuda_stream)
@@ -550,6 +551,23 @@ def calibrate(args) -> int:
         out.update(block="matrix wave: 8 dependent v_mfma_f32_32x32x16_f16 (256 cycles); vector wave: 48 v_fma_f32 + "
                          "16 v_exp_f32 on 16 independent values; one wave of each kind per SIMD, one workgroup per CU",
                    results=rows)
+    elif args.calib == "attnloop":
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        tiles = 1200
+        rows = []
+        for variant, name, qpw, per_cu in ((0, "32 queries per wave, 2 waves per SIMD (the kernel's shape)", 1, 2),
+                                           (1, "the same without the softmax", 1, 2),
+                                           (2, "64 queries per wave, 1 wave per SIMD, compiler's order", 2, 1),
+                                           (3, "64 queries per wave, one MFMA per six vector instructions (scheduling groups)", 2, 1),
+                                           (4, "64 queries per wave without the softmax", 2, 1)):
+            ms = timed(lambda: ok(lib.fl_calib_attn_loop(variant, cus, tiles, sink.data_ptr(), sp)), 2)
+            wave_tiles = cus * per_cu * 4 * tiles * qpw
+            rows.append({"variant": name, "us": round(ms * 1e3, 1),
+                         "TFLOPs": round(wave_tiles * 16 * 32768 / (ms * 1e-3) / 1e12, 1),
+                         "ns_per_32x32_tile_per_simd": round(ms * 1e6 / (wave_tiles / (4 * cus)), 1)})
+        out.update(loop="tile loop of prefill_attn_f16_kernel at D=128 on LDS-resident key tiles: per 32-query x 32-key tile "
+                        "16 x v_mfma_f32_32x32x16_f16 (512 matrix cycles), base-2 online softmax, 8 ds_read_b128 + 16 "
+                        "ds_read_b64_tr_b16, one workgroup barrier", results=rows)
     elif args.calib == "launch":
         ms = timed(lambda: ok(lib.fl_calib_empty(sp)), 2000)
         out.update(empty_kernel_us_per_launch=round(ms * 1e3, 3),
@@ -575,11 +593,12 @@ def main() -> int:
     ap.add_argument("--no-others", action="store_true",
                     help="skip the other_configs object (the remaining configurations, measured in the same run "
                          "with the headline workload)")
-    ap.add_argument("--calib", choices=["copy", "read", "mfma", "coexec", "launch"],
+    ap.add_argument("--calib", choices=["copy", "read", "mfma", "coexec", "attnloop", "launch"],
                     help="measurement-only legs, then exit.  copy: a plain 1 GiB -> 1 GiB elementwise copy (for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings); read: 2 GiB streaming read, plain and non-temporal "
                          "loads; mfma: register-only MFMA loops; coexec: a matrix wave and a vector wave per SIMD, alone and together, "
-                         "on a sixteenth of the CUs and on all of them; launch: empty-kernel launch cadence")
+                         "on a sixteenth of the CUs and on all of them; attnloop: the prompt-phase kernel's tile loop on LDS-resident tiles, "
+                         "with and without the softmax, 32 or 64 queries per wave; launch: empty-kernel launch cadence")
     ap.add_argument("--calib-copy", action="store_true", help="same as --calib copy")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
     ap.add_argument("--prefill-mask", default="causal", choices=["causal", "causal-1e5", "block-causal", "none"],

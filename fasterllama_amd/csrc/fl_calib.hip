@@ -9,6 +9,10 @@
 //   fl_calib_coexec        one wave of matrix work and one wave of vector (fma + exp2) work per SIMD, each alone
 //                          and both together, on a chosen number of CUs: how far the two pipes overlap, and
 //                          what chip-wide load does to the clock
+//   fl_calib_attn_loop     the tile loop of the fp16 prompt-phase attention kernel on key tiles that stay in LDS
+//                          (no global memory, no mask, no prologue or epilogue): what the loop's instruction mix
+//                          sustains by itself, with and without the softmax, at 32 queries per wave and two waves
+//                          per SIMD or 64 queries per wave and one, scheduling left to the compiler or forced
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -164,6 +168,182 @@ __global__ __launch_bounds__(512) void coexec_kernel(float *sink, int iters, int
     if (r == 123.456f) sink[0] = r;
 }
 
+
+typedef _Float16 half4c __attribute__((ext_vector_type(4)));
+typedef _Float16 half2c __attribute__((ext_vector_type(2)));
+typedef float float2c __attribute__((ext_vector_type(2)));
+typedef short short4c __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ half4c calib_read_tr16(const _Float16 *lds)
+{
+    typedef short4c __attribute__((address_space(3))) * lds_ptr;
+    return __builtin_bit_cast(half4c, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)lds));
+}
+
+__device__ __forceinline__ float calib_cross_half_max(float x)
+{
+    const unsigned u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+// The tile loop of prefill_attn_f16_kernel at D = 128 on three 32-key tiles (K 8 KB + V 8 KB each, the kernel's
+// swizzled layout) that are written to LDS once: per tile and 32-query sub-block 8 MFMAs S^T = K Q^T, the base-2
+// online softmax with its lazy rescale, 8 MFMAs O^T += V^T P^T, one workgroup barrier per tile.  QPW sub-blocks per
+// wave (1: as the kernel; 2: 64 queries per wave, the K and V operands read once for both).  SOFTMAX 0 replaces the
+// softmax by a conversion of the scores.  GROUPS (QPW = 2): the second sub-block's first product is issued between
+// the vector instructions of the first one's exponentials, and the first one's second product between those of the
+// second, one MFMA per GROUPS vector instructions (scheduling groups); 0 leaves the order to the compiler.
+template <int QPW, int SOFTMAX, int GROUPS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(QPW == 2 ? 1 : 2, QPW == 2 ? 1 : 2)))
+void attn_loop_kernel(float *sink, int tiles)
+{
+    constexpr int NC = 8, NDT = 4;
+    constexpr uint32_t kTileBytes = 16384, kVOff = 8192;
+    extern __shared__ __attribute__((aligned(16))) _Float16 smem[]; // sized by the host for the wanted workgroups per CU
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int qi = lane & 31, hf = lane >> 5;
+    for (int i = tid; i < 3 * 8192; i += 256) smem[i] = (_Float16)lane_value((uint32_t)i + blockIdx.x * 7919u, true);
+    __syncthreads();
+    half8 qreg[QPW][NC];
+#pragma unroll
+    for (int a = 0; a < QPW; ++a)
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) qreg[a][c][i] = (_Float16)(0.5f * lane_value(tid * 977u + a * 131u + c * 8 + i, true));
+    floatx16 ot[QPW][NDT];
+#pragma unroll
+    for (int a = 0; a < QPW; ++a)
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) ot[a][dt][v] = 0.f;
+    float m[QPW], l[QPW];
+#pragma unroll
+    for (int a = 0; a < QPW; ++a) { m[a] = -1e9f; l[a] = 0.f; }
+    const float scale = 0.0883883f * 1.44269504f;
+    const uint32_t k_swz = (uint32_t)(qi * 256 + ((hf ^ (qi & 15)) << 4));
+    const int vrow = 4 * hf + ((lane & 15) >> 2), vcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    const uint32_t v_swz = (uint32_t)(vrow * 256 + ((vrow & 3) << 6) + vcol * 2);
+
+    auto max_phase = [&](int a, const floatx16 &st) __attribute__((always_inline)) {
+        float r = fmaxf(fmaxf(st[0], st[1]), st[2]);
+#pragma unroll
+        for (int v = 3; v < 15; v += 2) r = fmaxf(fmaxf(r, st[v]), st[v + 1]);
+        const float mx = fmaxf(m[a], calib_cross_half_max(fmaxf(r, st[15])) * scale);
+        if (__ballot(mx > m[a] + 8.0f) != 0ull) {
+            const float alpha = __builtin_amdgcn_exp2f(m[a] - mx);
+            m[a] = mx;
+            l[a] *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) ot[a][dt][v] *= alpha;
+        }
+    };
+    auto exp_phase = [&](int a, const floatx16 &st, half8 (&pr)[2]) __attribute__((always_inline)) {
+        if constexpr (SOFTMAX) {
+            const float nm = -m[a];
+#pragma unroll
+            for (int v = 0; v < 16; v += 2) {
+                float2c e;
+                e[0] = __builtin_amdgcn_exp2f(fmaf(st[v], scale, nm));
+                e[1] = __builtin_amdgcn_exp2f(fmaf(st[v + 1], scale, nm));
+                const half2c h = __builtin_convertvector(e, half2c);
+                pr[v / 8][v % 8] = h[0];
+                pr[v / 8][v % 8 + 1] = h[1];
+                l[a] = __builtin_amdgcn_fdot2(h, half2c{(_Float16)1, (_Float16)1}, l[a], false);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { pr[0][i] = (_Float16)st[i]; pr[1][i] = (_Float16)st[8 + i]; }
+        }
+    };
+    auto groups = [&]() __attribute__((always_inline)) {
+        if constexpr (GROUPS > 0) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one matrix instruction
+                __builtin_amdgcn_sched_group_barrier(0x002, GROUPS, 0); // GROUPS vector instructions
+            }
+        }
+    };
+    auto tile = [&](auto buf_tag) __attribute__((always_inline)) {
+        constexpr int buf = decltype(buf_tag)::value;
+        __syncthreads();
+        asm volatile("" ::: "memory"); // nothing is hoisted out of the loop
+        half8 kall[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+            kall[c] = *reinterpret_cast<const half8 *>(reinterpret_cast<const char *>(smem) + (uint32_t)buf * kTileBytes + (k_swz ^ (uint32_t)(c << 5)));
+        half8 va[NDT][2];
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const char *base = reinterpret_cast<const char *>(smem) + (uint32_t)buf * kTileBytes + kVOff + (v_swz ^ (uint32_t)(dt << 6));
+                const half4c lo = calib_read_tr16(reinterpret_cast<const _Float16 *>(base + (uint32_t)(16 * u * 256)));
+                const half4c hi = calib_read_tr16(reinterpret_cast<const _Float16 *>(base + (uint32_t)((16 * u + 8) * 256)));
+                va[dt][u][0] = lo[0]; va[dt][u][1] = lo[1]; va[dt][u][2] = lo[2]; va[dt][u][3] = lo[3];
+                va[dt][u][4] = hi[0]; va[dt][u][5] = hi[1]; va[dt][u][6] = hi[2]; va[dt][u][7] = hi[3];
+            }
+        floatx16 st[QPW];
+        half8 pr[QPW][2];
+#pragma unroll
+        for (int a = 0; a < QPW; ++a)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) st[a][v] = 0.f;
+        auto first_product = [&](int a) __attribute__((always_inline)) {
+#pragma unroll
+            for (int c = 0; c < NC; ++c) st[a] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kall[c], qreg[a][c], st[a], 0, 0, 0);
+        };
+        auto second_product = [&](int a) __attribute__((always_inline)) {
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) ot[a][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[dt][u], pr[a][u], ot[a][dt], 0, 0, 0);
+        };
+        if constexpr (QPW == 1) {
+            first_product(0);
+            if constexpr (SOFTMAX) max_phase(0, st[0]);
+            exp_phase(0, st[0], pr[0]);
+            second_product(0);
+        } else {
+            first_product(0);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (SOFTMAX) max_phase(0, st[0]);
+            __builtin_amdgcn_sched_barrier(0);
+            first_product(QPW - 1);
+            exp_phase(0, st[0], pr[0]);
+            groups();
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (SOFTMAX) max_phase(QPW - 1, st[QPW - 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            second_product(0);
+            exp_phase(QPW - 1, st[QPW - 1], pr[QPW - 1]);
+            groups();
+            __builtin_amdgcn_sched_barrier(0);
+            second_product(QPW - 1);
+        }
+    };
+    for (int t = 0; t < tiles; t += 3) {
+        tile(std::integral_constant<int, 0>{});
+        tile(std::integral_constant<int, 1>{});
+        tile(std::integral_constant<int, 2>{});
+    }
+    float r = 0.f;
+#pragma unroll
+    for (int a = 0; a < QPW; ++a) {
+        r += l[a] + m[a];
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) r += ot[a][dt][v];
+    }
+    if (r == 123.456f) sink[0] = r;
+}
+
 } // namespace
 
 extern "C" {
@@ -219,6 +399,28 @@ int fl_calib_coexec(int what, int cus, int iters, float *sink, void *stream)
     if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL(coexec_kernel, dim3(cus), dim3(512), lds, static_cast<hipStream_t>(stream), sink, iters, what);
     return (int)hipGetLastError();
+}
+
+// The attention tile loop on LDS-resident tiles, 256 workgroups per CU-slot: variant 0 = 32 queries per wave, two
+// workgroups per CU (the kernel's shape); 1 = the same without the softmax; 2 = 64 queries per wave, one workgroup per
+// CU, compiler's order; 3 = the same with forced groups of one MFMA per six vector instructions; 4 = 64 queries per
+// wave without the softmax.  `tiles` must be a multiple of 3.  Useful FLOPs per launch:
+//   cus * wgs_per_cu * 4 waves * tiles * QPW * 16 MFMAs * 32768.
+int fl_calib_attn_loop(int variant, int cus, int tiles, float *sink, void *stream)
+{
+    if (!sink || cus <= 0 || tiles <= 0 || tiles % 3 != 0 || variant < 0 || variant > 4) return (int)hipErrorInvalidValue;
+    const int per_cu = variant <= 1 ? 2 : 1;
+    const int lds = per_cu == 1 ? 100 * 1024 : 64 * 1024; // dynamic LDS sized so that exactly per_cu workgroups fit a CU
+    const void *k = variant == 0   ? reinterpret_cast<const void *>(attn_loop_kernel<1, 1, 0>)
+                    : variant == 1 ? reinterpret_cast<const void *>(attn_loop_kernel<1, 0, 0>)
+                    : variant == 2 ? reinterpret_cast<const void *>(attn_loop_kernel<2, 1, 0>)
+                    : variant == 3 ? reinterpret_cast<const void *>(attn_loop_kernel<2, 1, 6>)
+                                   : reinterpret_cast<const void *>(attn_loop_kernel<2, 0, 0>);
+    hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return (int)e;
+    void *args[] = {&sink, &tiles};
+    e = hipLaunchKernel(k, dim3(cus * per_cu), dim3(256), args, lds, static_cast<hipStream_t>(stream));
+    return (int)(e != hipSuccess ? e : hipGetLastError());
 }
 
 } // extern "C"

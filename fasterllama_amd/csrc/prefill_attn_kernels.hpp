@@ -1031,8 +1031,6 @@ void prefill_attn_f16_kernel(const PrefillParams p)
         if constexpr (DMA) return lds_read_tr16(reinterpret_cast<const _Float16 *>(reinterpret_cast<const char *>(smem) + (uint32_t)buf * kTileBytes + kVOff + (uint32_t)(row0 * 256) + (v_swz ^ (uint32_t)(dt << 6))));
         else return lds_read_tr16(&sV[buf][row0 + vrow][32 * dt + vcol]);
     };
-    const float inv_scale = 1.0f / p.scale;
-    const float pair_raw = kPairLogit * inv_scale; // the remainder product's threshold in units of the raw products
     const bool mask_vec4 = HAS_MASK && (p.mask_ld & 3) == 0 && (reinterpret_cast<uintptr_t>(p.attn_mask) & 15u) == 0;
 
     // The rotated queries must have landed before the loop: a wait inside it would also wait for
@@ -1135,6 +1133,11 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 }
                 const half8 ka0 = kall[0];
                 if (special) {
+                    // (1 / scale is formed here, where it is needed: as a value kept across the loop it cost the
+                    // masked pair instance the registers it does not have)
+                    float sc = p.scale;
+                    asm volatile("" : "+v"(sc));
+                    const float inv_scale = 1.0f / sc;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         st[v] *= inv_scale;
@@ -1190,7 +1193,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 // typically, the size of the rounding of the weights to fp16 that every tile carries anyway.
                 float mxq = cross_half_max(max16(st)); // raw units
                 if constexpr (QSPLIT) {
-                    if (__ballot(!(fabsf(mxq) <= pair_raw)) != 0ull) {
+                    if (__ballot(!(fabsf(mxq * scale) <= kPairLogit * kLog2e)) != 0ull) { // (scale carries log2 e)
 #pragma unroll
                         for (int c = 0; c < NC; ++c) st = __builtin_amdgcn_mfma_f32_32x32x16_f16(kall[PF_KA ? c : 0], qlo[c], st, 0, 0, 0);
                         mxq = cross_half_max(max16(st));
@@ -1274,8 +1277,13 @@ void prefill_attn_f16_kernel(const PrefillParams p)
     if constexpr (DMA) asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // (a workgroup with an empty list never waited for its guessed tile)
     __syncthreads(); // every wave is done with the last K/V tile
     {
-        float *so = reinterpret_cast<float *>(smem) + wave * 32 * LDO;
-        const int q0 = qb * kPrefillQueriesPerBlock + wave * 32;
+        // The lane's place is derived again from the thread index here: values computed before the loop and used
+        // only after it would have to stay in registers across it (the masked pair instance has none to spare).
+        int tid_e = threadIdx.x;
+        asm volatile("" : "+v"(tid_e));
+        const int lane_e = tid_e & 63, wave_e = tid_e >> 6, qi_e = tid_e & 31, hf_e = (tid_e >> 5) & 1;
+        float *so = reinterpret_cast<float *>(smem) + wave_e * 32 * LDO;
+        const int q0 = qb * kPrefillQueriesPerBlock + wave_e * 32;
         float *dst0 = p.out + ((size_t)bh * S + q0) * D;
         constexpr int LPRW = HALF_D / 4;               // lanes per row when reading back
         constexpr int RPI = 64 / LPRW;                 // rows per store instruction
@@ -1286,7 +1294,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
                 const int dt = pass * (HALF_D / 32) + dd;
 #pragma unroll
                 for (int g4 = 0; g4 < 4; ++g4)
-                    *reinterpret_cast<float4 *>(so + qi * LDO + 32 * dd + 8 * g4 + 4 * hf) =
+                    *reinterpret_cast<float4 *>(so + qi_e * LDO + 32 * dd + 8 * g4 + 4 * hf_e) =
                         make_float4(ot[dt][4 * g4 + 0] * rl, ot[dt][4 * g4 + 1] * rl, ot[dt][4 * g4 + 2] * rl,
                                     ot[dt][4 * g4 + 3] * rl);
             }
@@ -1295,7 +1303,7 @@ void prefill_attn_f16_kernel(const PrefillParams p)
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
             for (int r0 = 0; r0 < 32; r0 += RPI) {
-                const int r = r0 + lane / LPRW, c4 = lane % LPRW;
+                const int r = r0 + lane_e / LPRW, c4 = lane_e % LPRW;
                 const float4 v = *reinterpret_cast<const float4 *>(so + r * LDO + 4 * c4);
                 if (q0 + r < S) *reinterpret_cast<float4 *>(dst0 + (size_t)r * D + pass * HALF_D + 4 * c4) = v;
             }
