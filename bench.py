@@ -685,7 +685,8 @@ def main() -> int:
         saved = (args.prefill_mask, args.prefill_fast_qk, args.prefill_classify_per_call)
         args.prefill_mask, args.prefill_fast_qk, args.prefill_classify_per_call = "causal", False, False
         for name in ("prefill_7b_b8_s1024", "prefill_7b_b8_s1024_f32", "prefill_7b_b1_s4096"):
-            others[name] = prefill_summary(measure_prefill(args, name, 20, 3, 3))
+            # (60 warm-up steps: the clock settles only after some 10 ms of matrix load; the first regions of a cold run read 10-15 % slow)
+            others[name] = prefill_summary(measure_prefill(args, name, 50, 60, 5))
         args.prefill_mask, args.prefill_fast_qk, args.prefill_classify_per_call = saved
         # OpenDecoder::forward under the reference driver's call pattern, at the small (B=1, ctx 4096) and the headline shape
         others["opendecoder_loop_cfg4"] = opendecoder_loop(1, 32, 128, 4096, 4095, 12, 20)
