@@ -41,6 +41,7 @@ EXPORTED_SYMBOLS = (
     "fl_decode_attn_workspace_init",
     "fl_prefill_attn_workspace_bytes",
     "fl_prefill_attn_forward",
+    "fl_prefill_attn_forward_passes",
     "fl_prefill_mask_classes_bytes",
     "fl_prefill_mask_classify",
     "fl_rope_table",
@@ -148,6 +149,8 @@ def load() -> C.CDLL:
     lib.fl_prefill_attn_workspace_bytes.restype = C.c_int
     lib.fl_prefill_attn_forward.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnIO), C.c_int32, C.c_void_p]
     lib.fl_prefill_attn_forward.restype = C.c_int
+    lib.fl_prefill_attn_forward_passes.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnIO), C.c_int32, C.c_void_p, C.c_int]
+    lib.fl_prefill_attn_forward_passes.restype = C.c_int
     lib.fl_prefill_mask_classes_bytes.argtypes = [C.POINTER(AttnDesc), C.POINTER(C.c_size_t)]
     lib.fl_prefill_mask_classes_bytes.restype = C.c_int
     lib.fl_prefill_mask_classify.argtypes = [C.POINTER(AttnDesc), C.c_void_p, C.c_int64, C.c_void_p, C.c_size_t, C.c_void_p]

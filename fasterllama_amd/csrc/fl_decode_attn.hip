@@ -375,7 +375,7 @@ PrefillWorkspace prefill_workspace(const fl_attn_desc *d, int S)
 }
 
 template <typename T, int D>
-hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
+hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream, int passes)
 {
     constexpr int VEC = flattn::Vec16<T>::N;
     constexpr int LPR = flattn::lanes_per_row(D / VEC);
@@ -386,15 +386,19 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
     const int hpt = std::is_same<T, _Float16>::value && !p.inp_scale && p.H % 4 == 0 ? 4 : 1;
     const int64_t groups = (int64_t)p.B * p.S * (p.H / hpt);
     const dim3 agrid((unsigned)((groups + ROWS - 1) / ROWS));
-    hipError_t e = hpt == 4 ? launch(flattn::prefill_rope_append_kernel<T, D, 4>, agrid, dim3(256), stream, p)
-                            : launch(flattn::prefill_rope_append_kernel<T, D, 1>, agrid, dim3(256), stream, p);
-    if (e != hipSuccess) return e;
+    hipError_t e = hipSuccess;
     const unsigned qblocks = (unsigned)((p.S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock);
-    if (p.attn_mask && !p.class_table) { // no table of the whole mask at hand: classify the rows of this call
-        const int ktiles = (p.start_pos + p.S + flattn::kPrefillKeysPerStep - 1) / flattn::kPrefillKeysPerStep;
-        e = launch(flattn::prefill_mask_classify_kernel, dim3((unsigned)ktiles, qblocks), dim3(256), stream, p, ktiles);
+    if (passes & 1) {
+        e = hpt == 4 ? launch(flattn::prefill_rope_append_kernel<T, D, 4>, agrid, dim3(256), stream, p)
+                     : launch(flattn::prefill_rope_append_kernel<T, D, 1>, agrid, dim3(256), stream, p);
         if (e != hipSuccess) return e;
+        if (p.attn_mask && !p.class_table) { // no table of the whole mask at hand: classify the rows of this call
+            const int ktiles = (p.start_pos + p.S + flattn::kPrefillKeysPerStep - 1) / flattn::kPrefillKeysPerStep;
+            e = launch(flattn::prefill_mask_classify_kernel, dim3((unsigned)ktiles, qblocks), dim3(256), stream, p, ktiles);
+            if (e != hipSuccess) return e;
+        }
     }
+    if (!(passes & 2)) return hipSuccess;
     if constexpr (prefill_wide(D)) {
         const unsigned qb32 = (unsigned)((p.S + flattn::kWideQueriesPerBlock - 1) / flattn::kWideQueriesPerBlock);
         const dim3 wgrid(qb32 * (unsigned)(p.B * p.H)), wblock(flattn::kWideWaves * 64);
@@ -415,16 +419,16 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream)
 }
 
 template <typename T>
-hipError_t dispatch_prefill(int D, const flattn::PrefillParams &p, hipStream_t stream)
+hipError_t dispatch_prefill(int D, const flattn::PrefillParams &p, hipStream_t stream, int passes)
 {
     switch (D) {
-    case 32: return launch_prefill<T, 32>(p, stream);
-    case 64: return launch_prefill<T, 64>(p, stream);
-    case 96: return launch_prefill<T, 96>(p, stream);
-    case 128: return launch_prefill<T, 128>(p, stream);
-    case 256: return launch_prefill<T, 256>(p, stream);
-    case 512: return launch_prefill<T, 512>(p, stream);
-    case 1024: return launch_prefill<T, 1024>(p, stream);
+    case 32: return launch_prefill<T, 32>(p, stream, passes);
+    case 64: return launch_prefill<T, 64>(p, stream, passes);
+    case 96: return launch_prefill<T, 96>(p, stream, passes);
+    case 128: return launch_prefill<T, 128>(p, stream, passes);
+    case 256: return launch_prefill<T, 256>(p, stream, passes);
+    case 512: return launch_prefill<T, 512>(p, stream, passes);
+    case 1024: return launch_prefill<T, 1024>(p, stream, passes);
     default: return hipErrorInvalidValue;
     }
 }
@@ -657,6 +661,12 @@ int fl_prefill_attn_workspace_bytes(const fl_attn_desc *desc, int32_t seq_len, s
 
 int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io_in, int32_t seq_len, void *hip_stream)
 {
+    return fl_prefill_attn_forward_passes(desc, io_in, seq_len, hip_stream, 3);
+}
+
+int fl_prefill_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io_in, int32_t seq_len, void *hip_stream, int passes)
+{
+    if (passes < 1 || passes > 3) return FL_ATTN_ERR_ARGUMENT;
     fl_attn_desc desc_copy;
     int st = import_desc(&desc, &desc_copy);
     if (st != FL_ATTN_OK) return st;
@@ -712,9 +722,9 @@ int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io_in, i
     p.fast_qk = (desc->flags & FL_ATTN_FLAG_FAST_PROMPT_QK) != 0;
 
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-    hipError_t e = desc->dtype == FL_ATTN_F16 ? dispatch_prefill<_Float16>(D, p, stream) : dispatch_prefill<float>(D, p, stream);
+    hipError_t e = desc->dtype == FL_ATTN_F16 ? dispatch_prefill<_Float16>(D, p, stream, passes) : dispatch_prefill<float>(D, p, stream, passes);
     if (!check_hip(e)) return FL_ATTN_ERR_HIP;
-    if (quant) {
+    if (quant && (passes & 2)) {
         if (!check_hip(launch(flattn::attn_quantize_transpose_kernel, dim3((unsigned)(desc->batch_size * seq_len)), dim3(flattn::kQuantThreads),
                               stream, p.out, io->out_int8, io->out_scale, desc->head_num, seq_len, D)))
             return FL_ATTN_ERR_HIP;

@@ -141,11 +141,15 @@ class PrefillAttention(DecodeAttention):
                                                          table.data_ptr(), table.numel(), C.c_void_p(s.cuda_stream)))
         return table
 
-    def launch_prefill(self, io: capi.AttnIO, seq_len: int, stream: torch.cuda.Stream | None = None) -> int:
+    def launch_prefill(self, io: capi.AttnIO, seq_len: int, stream: torch.cuda.Stream | None = None, passes: int = 3) -> int:
+        """passes: 1 = RoPE + append only, 2 = attention (+ INT8 epilogue) only, 3 = the whole step."""
         s = stream if stream is not None else torch.cuda.current_stream(self.device)
         with torch.cuda.device(self.device):
-            return self.lib.fl_prefill_attn_forward(C.byref(self.desc), C.byref(io), seq_len,
-                                                    C.c_void_p(s.cuda_stream))
+            if passes == 3:
+                return self.lib.fl_prefill_attn_forward(C.byref(self.desc), C.byref(io), seq_len,
+                                                        C.c_void_p(s.cuda_stream))
+            return self.lib.fl_prefill_attn_forward_passes(C.byref(self.desc), C.byref(io), seq_len,
+                                                           C.c_void_p(s.cuda_stream), passes)
 
     def prefill(self, q, k_new, v_new, k_cache, v_cache, freq_cis, start_pos: int = 0, out=None, **kw):
         d = self.desc

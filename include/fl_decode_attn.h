@@ -208,6 +208,15 @@ int fl_prefill_attn_workspace_bytes(const fl_attn_desc *desc, int32_t seq_len, s
 int fl_prefill_attn_forward(const fl_attn_desc *desc, const fl_attn_io *io, int32_t seq_len,
                             void *hip_stream);
 
+/* Same, restricted to some passes: bit 0 = RoPE + cache append of the new rows (and the per-call classification of
+ * the mask rows, where no class table is given), bit 1 = the attention kernel (and the optional INT8 epilogue) over
+ * the cache rows as they are.  Lets a profiler or benchmark time the matrix-core kernel alone: pass 2 after a pass
+ * 1 (or after a whole call) with the same operands recomputes the same output.  fl_prefill_attn_forward == passes 3.
+ * (Reference: the two halves are launchQKRoteEmbeddingTranspose / launchStoreKVcacheKernel, open_decoder.cu:142-177,
+ * and the GEMM - softmax - GEMM sequence, :179-228.) */
+int fl_prefill_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *io, int32_t seq_len,
+                                   void *hip_stream, int passes);
+
 /* The mask of the reference is one [L, L] array that every layer and every call reuses
  * (samples/llama_fp16.cu:139-150), so its 32 x 32 tiles can be classified (all <= -1e30 / all zero / the
  * diagonal tile of a causal mask / anything else) once: fl_prefill_mask_classify writes one byte per tile (fl_prefill_mask_classes_bytes bytes: key tile t, row

@@ -156,6 +156,8 @@ def test_workspace_validation_for_split_plans():
     assert lib.fl_decode_attn_forward(C.byref(d), C.byref(io), None) == capi.FL_ATTN_ERR_WORKSPACE
     assert lib.fl_decode_attn_forward_passes(C.byref(d), C.byref(fake_io()), None, 0) == capi.FL_ATTN_ERR_ARGUMENT
     assert lib.fl_decode_attn_forward_passes(C.byref(d), C.byref(fake_io()), None, 4) == capi.FL_ATTN_ERR_ARGUMENT
+    assert lib.fl_prefill_attn_forward_passes(C.byref(d), C.byref(fake_io()), 8, None, 0) == capi.FL_ATTN_ERR_ARGUMENT
+    assert lib.fl_prefill_attn_forward_passes(C.byref(d), C.byref(fake_io()), 8, None, 4) == capi.FL_ATTN_ERR_ARGUMENT
 
 
 def test_plans_cover_the_context_and_respect_forced_splits():

@@ -461,6 +461,37 @@ def test_prefill_with_a_persistent_mask_class_table(gpu, dtype, D):
     assert (np.diag(tab) == 3).all() and (tab[np.arange(4, 10), np.arange(0, 6)] == 0).all()
 
 
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_prefill_passes_append_then_attention_equals_one_call(gpu, dtype):
+    """fl_prefill_attn_forward_passes: pass 1 (RoPE + append, classification) followed by pass 2 (attention) gives the
+    bits of the whole call, pass 2 alone leaves the caches untouched, and a repeated pass 2 recomputes the same output."""
+    import torch
+    from fasterllama_amd.decode_attn import PrefillAttention
+    B, H, D, L, S, P = 2, 3, 128, 256, 150, 32
+    tdt = torch.float16 if dtype == "f16" else torch.float32
+    q, k, v, kc, vc, f = make(B, H, D, L, S, dtype, 5)
+    mask = causal_mask(L, -FMAX)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+    op = PrefillAttention(B, H, D, L, S, tdt, device=gpu)
+    qd, kd, vd, fd, md = t(q), t(k), t(v), t(f), t(mask)
+    kc1, vc1 = t(kc), t(vc)
+    whole = op.prefill(qd, kd, vd, kc1, vc1, fd, start_pos=P, attn_mask=md)
+    kc2, vc2 = t(kc), t(vc)
+    out = torch.full((B, H, S, D), float("nan"), dtype=torch.float32, device=gpu)
+    io = op.make_io(qd, kd, vd, kc2, vc2, fd, out, start_pos=P, attn_mask=md)
+    capi.check(op.launch_prefill(io, S, passes=1))
+    torch.cuda.synchronize()
+    assert torch.isnan(out).all()  # the append pass writes no output
+    assert torch.equal(kc2.view(torch.uint8), kc1.view(torch.uint8)) and torch.equal(vc2.view(torch.uint8), vc1.view(torch.uint8))
+    for _ in range(2):
+        out.fill_(float("nan"))
+        capi.check(op.launch_prefill(io, S, passes=2))
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int32), whole.view(torch.int32))
+        assert torch.equal(kc2.view(torch.uint8), kc1.view(torch.uint8))
+    assert op.launch_prefill(io, S, passes=0) == capi.FL_ATTN_ERR_ARGUMENT
+
+
 def test_prefill_argument_errors(gpu):
     import torch
     from fasterllama_amd.decode_attn import PrefillAttention
