@@ -1,6 +1,7 @@
 // C ABI of the decode-step attention library (see include/fl_decode_attn.h).
 // Host side: argument validation, launch planning and kernel dispatch.  Enqueue-only: no
-// allocation, no synchronisation, no state kept between calls.
+// allocation, no synchronisation; between calls the library remembers two immutable facts per device
+// (its compute unit count and the address of its scratch array) and nothing about the caller.
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -385,6 +386,7 @@ hipError_t launch_prefill(const flattn::PrefillParams &p, hipStream_t stream, in
     // nothing or lose: 71.2 -> 74.8 us)
     const int hpt = std::is_same<T, _Float16>::value && !p.inp_scale && p.H % 4 == 0 ? 4 : 1;
     const int64_t groups = (int64_t)p.B * p.S * (p.H / hpt);
+    if ((groups + ROWS - 1) / ROWS > (int64_t)INT32_MAX) return hipErrorInvalidValue; // one-dimensional grid
     const dim3 agrid((unsigned)((groups + ROWS - 1) / ROWS));
     hipError_t e = hipSuccess;
     const unsigned qblocks = (unsigned)((p.S + flattn::kPrefillQueriesPerBlock - 1) / flattn::kPrefillQueriesPerBlock);
@@ -694,7 +696,9 @@ int fl_prefill_attn_forward_passes(const fl_attn_desc *desc, const fl_attn_io *i
     if (io->rope_row < FL_ATTN_ROPE_AT_POSITION) return FL_ATTN_ERR_POSITION;
     if (io->attn_mask && (io->mask_ld < 0 || (io->mask_ld != 0 && io->mask_ld < (int64_t)io->start_pos + seq_len)))
         return FL_ATTN_ERR_ARGUMENT;
-    if ((int64_t)desc->batch_size * desc->head_num * ((seq_len + 31) / 32) > (int64_t)INT32_MAX) return FL_ATTN_ERR_SHAPE;
+    // one-dimensional grids: the attention kernels take a workgroup per 32 or 128 queries of a head, the append kernel
+    // one per 4 to 64 (token, head) rows
+    if ((int64_t)desc->batch_size * desc->head_num * ((seq_len + 3) / 4) > (int64_t)INT32_MAX) return FL_ATTN_ERR_SHAPE;
 
     const PrefillWorkspace wl = prefill_workspace(desc, seq_len);
     if (!io->workspace || io->workspace_bytes < wl.total) return FL_ATTN_ERR_WORKSPACE;

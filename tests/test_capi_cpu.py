@@ -160,6 +160,14 @@ def test_workspace_validation_for_split_plans():
     assert lib.fl_prefill_attn_forward_passes(C.byref(d), C.byref(fake_io()), 8, None, 4) == capi.FL_ATTN_ERR_ARGUMENT
 
 
+def test_prompt_grids_that_exceed_the_launch_limit_are_a_shape_error():
+    """B * H * ceil(S / 4) workgroups of the append kernel must fit a one-dimensional grid."""
+    lib = capi.load()
+    d = desc(B=2047, H=1024, D=32, L=8192, dtype=capi.FL_ATTN_F16)
+    assert lib.fl_prefill_attn_forward(C.byref(d), C.byref(fake_io(start_pos=0)), 8192, None) == capi.FL_ATTN_ERR_SHAPE
+    assert lib.fl_prefill_attn_forward(C.byref(d), C.byref(fake_io(workspace=None)), 64, None) == capi.FL_ATTN_ERR_WORKSPACE
+
+
 def test_plans_cover_the_context_and_respect_forced_splits():
     lib = capi.load()
     plan = capi.AttnPlan()
