@@ -95,9 +95,9 @@ def assert_cache_bit_exact(got, want, what=""):
     assert bad.size == 0, f"{what}: {bad.size} cache words differ, first at flat index {bad[:5]}"
 
 
-F32_REL_TOL = 1e-5      # north star: FP32 within 1e-5 relative
+F32_REL_TOL = 1e-5      # the bar for FP32 storage: within 1e-5 relative
 F32_ROW_FLOOR = 0.1     # ... of max(|ref|, 0.1 * largest |ref| of the same (b, h[, s]) output row)
-F16_ABS_TOL = 2e-3      # north star: fp16 storage within 2e-3 absolute
+F16_ABS_TOL = 2e-3      # the bar for fp16 storage: within 2e-3 absolute
 F32_VS_FLOAT_REF = 1.0   # see assert_out_close
 
 
