@@ -696,7 +696,8 @@ def main() -> int:
         o_steps, o_rep = max(10, min(args.steps, 50)), max(3, min(args.repeats, 3))
         for key, name, mask in (("cfg1", "cfg1", "none"), ("cfg2", "cfg2", "none"), ("cfg4", "cfg4", "none"),
                                 ("cfg5", "cfg5", "none"), ("cfg3_causal_mask", "cfg3", "causal"),
-                                ("cfg3_strict_mask", "cfg3", "strict")):
+                                ("cfg3_strict_mask", "cfg3", "strict"),
+                                ("cfg3_f32_caches", "x7b_f32", "none")):  # the headline shape in the reference's cache type
             others[key] = summary(measure_decode(name, args, o_steps, max(3, args.warmup // 2), o_rep, mask=mask))
         # the prompt phase of the same block (matrix-core bound: another roofline), reference driver's causal mask
         saved = (args.prefill_mask, args.prefill_fast_qk, args.prefill_classify_per_call)
